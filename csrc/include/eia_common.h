@@ -64,3 +64,11 @@ enum EiaStatus : int {
 #define EIA_LAUNCH_CHECK() return (int)hipGetLastError()
 
 #define EIA_API extern "C" __attribute__((visibility("default")))
+
+// Element access for kernels templated on the activation type (bf16 or float); math is fp32.
+template <typename T> EIA_DEV float ld_f32(const T* p, long i);
+template <> EIA_DEV float ld_f32<bf16_t>(const bf16_t* p, long i) { return (float)p[i]; }
+template <> EIA_DEV float ld_f32<float>(const float* p, long i) { return p[i]; }
+template <typename T> EIA_DEV void st_f32(T* p, long i, float v);
+template <> EIA_DEV void st_f32<bf16_t>(bf16_t* p, long i, float v) { p[i] = (bf16_t)v; }
+template <> EIA_DEV void st_f32<float>(float* p, long i, float v) { p[i] = v; }

@@ -88,3 +88,24 @@ EIA_API int eia_act(void* out, const void* x, long numel, int kind, hipStream_t 
   }
   EIA_LAUNCH_CHECK();
 }
+
+// Squared ReLU, out = max(x, 0)^2, for bf16 or fp32 activations (ungated expert MLPs).
+template <typename T>
+__global__ void __launch_bounds__(256)
+relu2_kernel(T* __restrict__ out, const T* __restrict__ x, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    const float v = fmaxf(ld_f32<T>(x, i), 0.f);
+    st_f32<T>(out, i, v * v);
+  }
+}
+
+EIA_API int eia_relu2(void* out, const void* x, long numel, int is_bf16, hipStream_t st) {
+  if (numel < 0) return EIA_BAD_SHAPE;
+  if (numel == 0) return EIA_OK;
+  dim3 grid(grid_for((numel + 3) / 4)), block(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(relu2_kernel<bf16_t>, grid, block, 0, st, (bf16_t*)out, (const bf16_t*)x, numel);
+  else
+    hipLaunchKernelGGL(relu2_kernel<float>, grid, block, 0, st, (float*)out, (const float*)x, numel);
+  EIA_LAUNCH_CHECK();
+}

@@ -524,3 +524,85 @@ EIA_API int eia_moe_combine_sk(const float* part, int sk, int rows, const float*
                      inv, k, H, static_cast<bf16_t*>(out), ldo);
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Group-limited sigmoid routing: logits z = W_r x in fp32, scores s = sigmoid(z); the experts
+// form `ngroups` equal groups of neighbours, a group scores the sum of its two largest s, only
+// experts of the `keep` best groups are eligible, the `k` largest eligible scores win and weigh
+// s * route_scale (not renormalised).  Ties go to the lower index.  One wave per token: lanes
+// split the width for the dot products, lane 0 selects (E <= 256).
+template <typename T>
+__global__ void __launch_bounds__(256)
+route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr, int H, int T_,
+                     int E, int k, int ngroups, int keep, float route_scale,
+                     float* __restrict__ tw, int* __restrict__ ids,
+                     const int* __restrict__ row_len) {
+  __shared__ float sc[4][256];
+  __shared__ unsigned char ok[4][256];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T_) return;
+  const T* xr = x + (long)t * ldx;
+  for (int e = 0; e < E; ++e) {
+    const T* w = wr + (long)e * H;
+    float p = 0.f;
+    for (int c = lane; c < H; c += 64) p += ld_f32<T>(xr, c) * ld_f32<T>(w, c);
+    p = wave_sum(p);
+    if (lane == 0) sc[wave][e] = 1.0f / (1.0f + expf(-p));
+  }
+  if (lane != 0) return;
+  float* s = sc[wave];
+  unsigned char* el = ok[wave];
+  const bool pad = row_len && row_len[t] == 0;
+  const int per = E / ngroups;
+  // group scores in place of a separate array: pick `keep` groups one by one
+  for (int e = 0; e < E; ++e) el[e] = 0;
+  for (int r = 0; r < keep; ++r) {
+    int best = -1;
+    float bv = 0.f;
+    for (int g = 0; g < ngroups; ++g) {
+      if (el[g * per]) continue;            // group already taken (its first expert is marked)
+      float m1 = -INFINITY, m2 = -INFINITY;
+      for (int e = g * per; e < (g + 1) * per; ++e) {
+        const float v = s[e];
+        if (v > m1) { m2 = m1; m1 = v; } else if (v > m2) m2 = v;
+      }
+      const float gs = m1 + (per > 1 ? m2 : 0.f);
+      if (best < 0 || gs > bv) { best = g; bv = gs; }
+    }
+    if (best < 0) break;
+    for (int e = best * per; e < (best + 1) * per; ++e) el[e] = 1;
+  }
+  for (int r = 0; r < k; ++r) {
+    int best = -1;
+    float bv = 0.f;
+    for (int e = 0; e < E; ++e)
+      if (el[e] == 1 && (best < 0 || s[e] > bv)) { best = e; bv = s[e]; }
+    if (best < 0 || pad) {
+      ids[(long)t * k + r] = E;             // routes nowhere
+      tw[(long)t * k + r] = 0.f;
+    } else {
+      el[best] = 2;
+      ids[(long)t * k + r] = best;
+      tw[(long)t * k + r] = bv * route_scale;
+    }
+  }
+}
+
+// x [T, H] (row stride ldx) and wr [E, H] in bf16 (is_bf16) or fp32 -> tw fp32 [T, k], ids [T, k].
+EIA_API int eia_moe_route_grouped(const void* x, long ldx, const void* wr, int H, int T, int E,
+                                  int k, int ngroups, int keep, float route_scale, float* tw,
+                                  int* ids, const int* row_len, int is_bf16, hipStream_t st) {
+  if (E < 1 || E > 256 || k < 1 || ngroups < 1 || E % ngroups || keep < 1 || keep > ngroups ||
+      k > keep * (E / ngroups))
+    return EIA_BAD_SHAPE;
+  if (T <= 0) return EIA_OK;
+  dim3 grid((T + 3) / 4), block(256);
+  if (is_bf16)
+    hipLaunchKernelGGL((route_grouped_kernel<bf16_t>), grid, block, 0, st, (const bf16_t*)x, ldx,
+                       (const bf16_t*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len);
+  else
+    hipLaunchKernelGGL((route_grouped_kernel<float>), grid, block, 0, st, (const float*)x, ldx,
+                       (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len);
+  EIA_LAUNCH_CHECK();
+}

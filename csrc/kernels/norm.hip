@@ -196,3 +196,65 @@ EIA_API int eia_layer_norm(void* out, const void* x, void* residual, const void*
 #undef LN_CASE
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Post-norm residual with an fp32 residual stream (sublayer-output norm):
+//   x[row] += layernorm(y[row]) * w          (no bias; variance = mean of squared deviations)
+//   xb[row] = (T) x[row]                      (optional copy in the activation type for the GEMMs)
+// and the plain form on an fp32 input:  out[row] = (T)(layernorm(x[row]) * w).
+// One workgroup per row, three passes over a row that stays in L1/L2 (mean, variance, write):
+// the two-pass variance keeps fp32 exact enough for widths of several thousand.
+template <typename TIn, typename T, bool RESID>
+__global__ void __launch_bounds__(256)
+ln_nobias_kernel(const TIn* __restrict__ y, long ldy, const T* __restrict__ w,
+                 float* __restrict__ x, T* __restrict__ out, long ldo, float eps, int W) {
+  __shared__ float scratch[4];
+  const long row = blockIdx.x;
+  const TIn* yr = y + row * ldy;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) s += ld_f32<TIn>(yr, c);
+  const float mean = block_sum(s, scratch) / (float)W;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float d = ld_f32<TIn>(yr, c) - mean;
+    q += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(q, scratch) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = (ld_f32<TIn>(yr, c) - mean) * inv * ld_f32<T>(w, c);
+    if constexpr (RESID) {
+      v += x[row * (long)W + c];
+      x[row * (long)W + c] = v;
+    }
+    if (out) st_f32<T>(out + row * ldo, c, v);
+  }
+}
+
+// y [rows, W] (bf16 when is_bf16 else fp32, row stride ldy); x fp32 [rows, W] contiguous, updated
+// in place; xb nullable copy of the new x in y's type.
+EIA_API int eia_ln_residual(const void* y, long ldy, const void* w, float* x, void* xb, long ldxb,
+                            float eps, int rows, int W, int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1) return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  if (is_bf16)
+    hipLaunchKernelGGL((ln_nobias_kernel<bf16_t, bf16_t, true>), dim3(rows), dim3(256), 0, st,
+                       (const bf16_t*)y, ldy, (const bf16_t*)w, x, (bf16_t*)xb, ldxb, eps, W);
+  else
+    hipLaunchKernelGGL((ln_nobias_kernel<float, float, true>), dim3(rows), dim3(256), 0, st,
+                       (const float*)y, ldy, (const float*)w, x, (float*)xb, ldxb, eps, W);
+  EIA_LAUNCH_CHECK();
+}
+
+// out [rows, W] (bf16 when is_bf16 else fp32) = layernorm(x fp32 [rows, W], row stride ldx) * w.
+EIA_API int eia_ln_f32in(const float* x, long ldx, const void* w, void* out, long ldo, float eps,
+                         int rows, int W, int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1 || !out) return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  if (is_bf16)
+    hipLaunchKernelGGL((ln_nobias_kernel<float, bf16_t, false>), dim3(rows), dim3(256), 0, st, x,
+                       ldx, (const bf16_t*)w, nullptr, (bf16_t*)out, ldo, eps, W);
+  else
+    hipLaunchKernelGGL((ln_nobias_kernel<float, float, false>), dim3(rows), dim3(256), 0, st, x,
+                       ldx, (const float*)w, nullptr, (float*)out, ldo, eps, W);
+  EIA_LAUNCH_CHECK();
+}

@@ -1,0 +1,174 @@
+// Linear-attention recurrence with per-channel data-dependent decay (RWKV-style "wkv" mixing)
+// on per-sequence state slots.
+//
+// State of a sequence and layer: S [heads, dk, dv] fp32 and the previous token's layer input
+// prev [width] fp32.  A sequence whose first scheduled position is 0 starts from zeros whatever
+// its slot held before, so slots are reused without clearing.
+//
+//   eia_token_shift_mix : mix_s[t] = x[t] + (x[t-1] - x[t]) * mu_s  for NS streams (x[-1] from
+//                         the slot; zeros at position 0)
+//   eia_wkv_scan        : w = exp(-exp(dec + w0));  o = (S + diag(u) k v^T)^T r;
+//                         S = diag(w) S + k v^T;  y = o / rms(o) * norm_w * silu(g)
+//                         and prev <- x[last token of the step]
+//
+// Batch layout: sequence s owns rows [cu[s], cu[s+1]) (cu == nullptr: row s).  All recurrence
+// math is fp32; activations are bf16 or fp32 (template T).
+#include "eia_common.h"
+
+EIA_DEV int find_seq(const int* cu, int nseq, int row) {
+  int lo = 0, hi = nseq - 1;               // largest s with cu[s] <= row
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu[mid] <= row) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+token_shift_mix_kernel(const float* __restrict__ x, const T* __restrict__ mu, int NS,
+                       const float* __restrict__ prev_state, const int* __restrict__ slots,
+                       const int* __restrict__ cu, int nseq, const int* __restrict__ positions,
+                       T* __restrict__ out, long out_ss, int W) {
+  const int row = blockIdx.x;
+  const int s = cu ? find_seq(cu, nseq, row) : row;
+  const int first = cu ? cu[s] : row;
+  const float* cur = x + (long)row * W;
+  const float* prv = nullptr;
+  if (row > first) prv = cur - W;
+  else if (positions[row] > 0 && slots[s] >= 0) prv = prev_state + (long)slots[s] * W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float a = cur[c];
+    const float d = (prv ? prv[c] : 0.f) - a;
+    for (int k = 0; k < NS; ++k)
+      st_f32<T>(out + (long)k * out_ss + (long)row * W, c, a + d * ld_f32<T>(mu, (long)k * W + c));
+  }
+}
+
+// x fp32 [rows, W]; mu [NS, W]; out [NS, rows, W] (stream stride out_ss elements).
+EIA_API int eia_token_shift_mix(const float* x, const void* mu, int NS, const float* prev_state,
+                                const int* slots, const int* cu, int nseq, const int* positions,
+                                void* out, long out_ss, int rows, int W, int is_bf16,
+                                hipStream_t st) {
+  if (rows < 0 || W < 1 || NS < 1 || nseq < 1) return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  if (is_bf16)
+    hipLaunchKernelGGL((token_shift_mix_kernel<bf16_t>), dim3(rows), dim3(256), 0, st, x,
+                       (const bf16_t*)mu, NS, prev_state, slots, cu, nseq, positions,
+                       (bf16_t*)out, out_ss, W);
+  else
+    hipLaunchKernelGGL((token_shift_mix_kernel<float>), dim3(rows), dim3(256), 0, st, x,
+                       (const float*)mu, NS, prev_state, slots, cu, nseq, positions, (float*)out,
+                       out_ss, W);
+  EIA_LAUNCH_CHECK();
+}
+
+struct WkvArgs {
+  const void *r, *k, *v, *g; long ld;       // [rows, H*D] each, row stride ld
+  const float* dec; long ld_dec;            // [rows, H*D] fp32 decay pre-activation (without w0)
+  const void *w0, *u, *norm_w;              // [H*D] each
+  float* S;                                 // [slots, H, D, D]
+  float* prev; const float* x; int W;       // prev [slots, W]; x fp32 [rows, W]
+  const int* slots; const int* cu; const int* positions; const int* seq_lens;
+  void* y; long ldy;                        // [rows, H*D]
+  float eps; int H, D;
+};
+
+// One workgroup per (sequence, head); thread j owns column j of S (dk values in registers,
+// DMAX >= D) and walks the sequence's tokens in order.
+template <typename T, int DMAX>
+__global__ void __launch_bounds__(DMAX < 64 ? 64 : DMAX)
+wkv_scan_kernel(WkvArgs a) {
+  __shared__ float sr[DMAX], sk[DMAX], sw[DMAX], su[DMAX], red[4];
+  const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x, D = a.D;
+  const int slot = a.slots[s];
+  if (slot < 0 || (a.seq_lens && a.seq_lens[s] <= 0)) return;
+  const int lo = a.cu ? a.cu[s] : s, hi = a.cu ? a.cu[s + 1] : s + 1;
+  if (hi <= lo) return;
+  const bool fresh = a.positions[lo] == 0;
+  float* Sg = a.S + ((long)slot * a.H + h) * D * D;
+  float S[DMAX];
+#pragma unroll
+  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && i < D && j < D) ? Sg[(long)i * D + j] : 0.f;
+  const long hc = (long)h * D;
+  if (j < D) su[j] = ld_f32<T>(static_cast<const T*>(a.u), hc + j);
+  const float w0 = j < D ? ld_f32<T>(static_cast<const T*>(a.w0), hc + j) : 0.f;
+  const float nw = j < D ? ld_f32<T>(static_cast<const T*>(a.norm_w), hc + j) : 0.f;
+  const T* R = static_cast<const T*>(a.r);
+  const T* K = static_cast<const T*>(a.k);
+  const T* V = static_cast<const T*>(a.v);
+  const T* G = static_cast<const T*>(a.g);
+  T* Y = static_cast<T*>(a.y);
+  for (int row = lo; row < hi; ++row) {
+    __syncthreads();
+    float vj = 0.f;
+    if (j < D) {
+      sr[j] = ld_f32<T>(R, row * a.ld + hc + j);
+      sk[j] = ld_f32<T>(K, row * a.ld + hc + j);
+      sw[j] = expf(-expf(a.dec[row * a.ld_dec + hc + j] + w0));
+      vj = ld_f32<T>(V, row * a.ld + hc + j);
+    }
+    __syncthreads();
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i) {
+      if (i < D) {
+        const float kv = sk[i] * vj;
+        o += sr[i] * (S[i] + su[i] * kv);
+        S[i] = sw[i] * S[i] + kv;
+      }
+    }
+    // head RMS norm over the D outputs, then channel weight and gate
+    float ss = wave_sum(j < D ? o * o : 0.f);
+    if (DMAX > 64) {
+      if ((j & 63) == 0) red[j >> 6] = ss;
+      __syncthreads();
+      ss = 0.f;
+      for (int q = 0; q < (DMAX + 63) / 64; ++q) ss += red[q];
+    }
+    if (j < D) {
+      const float gv = ld_f32<T>(G, row * a.ld + hc + j);
+      const float gate = gv / (1.0f + expf(-gv));
+      st_f32<T>(Y, row * a.ldy + hc + j, o / sqrtf(ss / (float)D + a.eps) * nw * gate);
+    }
+  }
+  if (j < D) {
+#pragma unroll
+    for (int i = 0; i < DMAX; ++i)
+      if (i < D) Sg[(long)i * D + j] = S[i];
+  }
+  if (h == 0) {
+    const float* last = a.x + (long)(hi - 1) * a.W;
+    float* p = a.prev + (long)slot * a.W;
+    for (int c = j; c < a.W; c += blockDim.x) p[c] = last[c];
+  }
+}
+
+EIA_API int eia_wkv_scan(const void* r, const void* k, const void* v, const void* g, long ld,
+                         const float* dec, long ld_dec, const void* w0, const void* u,
+                         const void* norm_w, float* S, float* prev, const float* x, int W,
+                         const int* slots, const int* cu, const int* positions,
+                         const int* seq_lens, void* y, long ldy, float eps, int nseq, int H, int D,
+                         int is_bf16, hipStream_t st) {
+  if (nseq < 0 || H < 1 || D < 1 || W < 1) return EIA_BAD_SHAPE;
+  if (D > 256) return EIA_UNSUPPORTED;
+  if (nseq == 0) return EIA_OK;
+  WkvArgs a{r, k, v, g, ld, dec, ld_dec, w0, u, norm_w, S, prev, x, W, slots, cu, positions,
+            seq_lens, y, ldy, eps, H, D};
+  dim3 grid(nseq, H);
+#define WKV_LAUNCH(TT, DM)                                                                 \
+  hipLaunchKernelGGL((wkv_scan_kernel<TT, DM>), grid, dim3(DM < 64 ? 64 : DM), 0, st, a)
+  if (is_bf16) {
+    if (D <= 32) WKV_LAUNCH(bf16_t, 32);
+    else if (D <= 64) WKV_LAUNCH(bf16_t, 64);
+    else if (D <= 128) WKV_LAUNCH(bf16_t, 128);
+    else WKV_LAUNCH(bf16_t, 256);
+  } else {
+    if (D <= 32) WKV_LAUNCH(float, 32);
+    else if (D <= 64) WKV_LAUNCH(float, 64);
+    else if (D <= 128) WKV_LAUNCH(float, 128);
+    else WKV_LAUNCH(float, 256);
+  }
+#undef WKV_LAUNCH
+  EIA_LAUNCH_CHECK();
+}

@@ -64,6 +64,16 @@ _SIGNATURES = {
     "eia_splitk_reduce": [P, I, I, I, P, P, L, S],
     "eia_splitk_swiglu": [P, I, I, I, P, L, S],
     "eia_splitk_add_rmsnorm": [P, I, I, I, P, P, F, P, L, S],
+    "eia_ln_residual": [P, L, P, P, P, L, F, I, I, I, S],
+    "eia_ln_f32in": [P, L, P, P, L, F, I, I, I, S],
+    "eia_latent_prep": [P, L, I, I, P, P, L, I, I, P, I, I, I, P, IP, IP, P, L, F, I, I, S],
+    "eia_latent_attn": [P, L, L, P, L, L, P, I, P, L, IP, I, IP, IP, IP, I, IP, P, L, P, L, L, F,
+                        I, I, I, I, I, I, S],
+    "eia_token_shift_mix": [P, P, I, P, IP, IP, I, IP, P, L, I, I, I, S],
+    "eia_wkv_scan": [P, P, P, P, L, P, L, P, P, P, P, P, P, I, IP, IP, IP, IP, P, L, F, I, I, I,
+                     I, S],
+    "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, S],
+    "eia_relu2": [P, P, L, I, S],
     "eia_ar_alloc": [P, L],
     "eia_moe_splitk_norm_route": [P, I, I, I, P, P, F, P, L, P, I, I, I, I, P, P, P, S],
     "eia_moe_combine_norm": [P, I, I, P, P, I, I, I, P, P, F, P, L, S],

@@ -41,6 +41,22 @@ def parse_dtype(name: str | torch.dtype) -> torch.dtype:
         raise ValueError(f"unsupported dtype {name!r}") from e
 
 
+def safetensors_shapes(path: str) -> Dict[str, Any]:
+    """name -> shape of every tensor in the *.safetensors files of a folder, from their headers
+    (8-byte little-endian length, then that many bytes of JSON); no tensor data is read."""
+    import glob
+    import struct
+    out: Dict[str, Any] = {}
+    for f in sorted(glob.glob(os.path.join(path, "*.safetensors"))):
+        with open(f, "rb") as fh:
+            (n,) = struct.unpack("<Q", fh.read(8))
+            hdr = json.loads(fh.read(n))
+        for k, v in hdr.items():
+            if k != "__metadata__":
+                out[k] = list(v["shape"])
+    return out
+
+
 @dataclasses.dataclass
 class ModelConfig:
     """Architecture hyper-parameters (a normalised view over an HF config.json)."""
@@ -120,7 +136,33 @@ class ModelConfig:
         return L * (attn + mlp + 2 * h) + emb
 
     @classmethod
+    def from_layer_list(cls, d: Dict[str, Any], name: str = "",
+                        tensor_shapes: Optional[Dict[str, Any]] = None) -> "ModelConfig":
+        """Designs whose config.json names the architecture in one string and lists the layers
+        one by one (Sekolorn): keys ``architecture``, ``vocab``, ``width``, ``norm.eps`` and
+        ``layers`` (kept whole in ``extra["layers"]``).  Sizes the file leaves to the checkpoint
+        (the rank of a wkv layer's decay branch) come from ``tensor_shapes`` when given."""
+        import copy
+        layers = copy.deepcopy(d["layers"])
+        for i, L in enumerate(layers):
+            m = L.setdefault("mixer", {})
+            if L.get("type") == "wkv" and "decay_rank" not in m:
+                shp = (tensor_shapes or {}).get(f"l{i}.mix.w1")
+                m["decay_rank"] = int(shp[0]) if shp else 64
+        heads = [L["mixer"].get("heads", 1) for L in layers]
+        eps = float((d.get("norm") or {}).get("eps", 1e-6))
+        return cls(architecture=d["architecture"], hidden_size=int(d["width"]),
+                   num_hidden_layers=len(layers), num_attention_heads=max(heads + [1]),
+                   vocab_size=int(d["vocab"]), num_key_value_heads=1,
+                   head_dim=max([L["mixer"].get("dim", 1) for L in layers] + [1]),
+                   max_position_embeddings=1 << 20,      # the design sets no limit
+                   rms_norm_eps=eps, layer_norm_eps=eps,
+                   name=name, extra={"layers": layers})
+
+    @classmethod
     def from_hf_dict(cls, d: Dict[str, Any], name: str = "") -> "ModelConfig":
+        if isinstance(d.get("architecture"), str) and isinstance(d.get("layers"), list):
+            return cls.from_layer_list(d, name)
         arch = (d.get("architectures") or [d.get("model_type", "LlamaForCausalLM")])[0]
         text = d.get("text_config")
         outer = d
@@ -193,7 +235,10 @@ class ModelConfig:
     @classmethod
     def from_pretrained(cls, path: str) -> "ModelConfig":
         with open(os.path.join(path, "config.json")) as f:
-            return cls.from_hf_dict(json.load(f), name=path)
+            d = json.load(f)
+        if isinstance(d.get("architecture"), str) and isinstance(d.get("layers"), list):
+            return cls.from_layer_list(d, name=path, tensor_shapes=safetensors_shapes(path))
+        return cls.from_hf_dict(d, name=path)
 
 
 @dataclasses.dataclass
@@ -205,6 +250,9 @@ class CacheConfig:
     swap_space_gb: float = 4.0               # --swap-space: pinned host KV for preemption
     enable_prefix_caching: bool = True
     cache_dtype: Optional[torch.dtype] = None   # None -> model dtype
+    # per-sequence state slots of recurrent layers (0: the model has none); set by EngineConfig
+    # to max_num_seqs for models that need them, which also turns prefix caching off
+    num_state_slots: int = 0
 
     def __post_init__(self) -> None:
         if self.block_size % 16 != 0 or self.block_size <= 0:
@@ -277,7 +325,9 @@ class EngineConfig:
     engine_iteration_timeout_s: float = 120.0  # VLLM_ENGINE_ITERATION_TIMEOUT_S
 
     def __post_init__(self) -> None:
-        if self.device == "cuda" and self.dtype != torch.bfloat16:
+        if self.device == "cuda" and self.dtype == torch.float32 and self._model_has_fp32_kernels():
+            pass        # this model's kernels have fp32 forms (true fp32 matrix products)
+        elif self.device == "cuda" and self.dtype != torch.bfloat16:
             # the HIP kernels (attention, norms, GEMM epilogues, sampling) are bf16-only; any
             # other dtype would silently run the PyTorch reference ops on the GPU
             raise ValueError(f"dtype {self.dtype} is not supported on the MI355X path; serve "
@@ -289,12 +339,24 @@ class EngineConfig:
             self.enforce_eager = True        # host-staged gloo collectives cannot be captured
         if self.cache.cache_dtype is None:
             self.cache.cache_dtype = self.dtype
+        if self._model_attr("needs_state_slots") and not self.cache.num_state_slots:
+            self.cache.num_state_slots = self.scheduler.max_num_seqs
         if self.scheduler.max_model_len > self.model.max_position_embeddings and \
                 os.environ.get("VLLM_ALLOW_LONG_MAX_MODEL_LEN", "0") not in ("1", "true", "True"):
             # Match vLLM behaviour: clamp unless explicitly allowed.
             self.scheduler.max_model_len = self.model.max_position_embeddings
         if self.scheduler.max_num_batched_tokens < self.scheduler.max_num_seqs:
             self.scheduler.max_num_batched_tokens = self.scheduler.max_num_seqs
+
+    def _model_attr(self, name: str) -> bool:
+        from .models import get_model_class
+        try:
+            return bool(getattr(get_model_class(self.model.architecture), name, False))
+        except ValueError:
+            return False
+
+    def _model_has_fp32_kernels(self) -> bool:
+        return self._model_attr("supports_float32")
 
     @property
     def max_blocks_per_seq(self) -> int:

@@ -8,14 +8,52 @@ from .. import _native
 from .sequence import Sequence
 
 
+class StateSlots:
+    """Fixed pool of per-sequence state slots (recurrent layers keep one state per live
+    sequence).  A slot is taken at admission and given back with the sequence's blocks; lowest
+    free slot first, so a freed slot is the next one handed out."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free = list(range(num_slots - 1, -1, -1))     # pop() yields the lowest
+        self._owner = {}                                     # seq_id -> slot
+
+    def slot_of(self, seq_id: int) -> int:
+        return self._owner.get(seq_id, -1)
+
+    def acquire(self, seq_id: int) -> int:
+        """The sequence's slot, newly taken if it had none; -1 when the pool is empty."""
+        s = self._owner.get(seq_id)
+        if s is not None:
+            return s
+        if not self._free:
+            return -1
+        s = self._free.pop()
+        self._owner[seq_id] = s
+        return s
+
+    def release(self, seq_id: int) -> None:
+        s = self._owner.pop(seq_id, None)
+        if s is not None:
+            self._free.append(s)
+            self._free.sort(reverse=True)
+
+    def num_free(self) -> int:
+        return len(self._free)
+
+
 class BlockManager:
-    def __init__(self, num_blocks: int, block_size: int, prefix_caching: bool = True):
+    def __init__(self, num_blocks: int, block_size: int, prefix_caching: bool = True,
+                 num_state_slots: int = 0):
         rt = _native.runtime()
+        # a cached prefix skips its tokens, but a recurrent state cannot be skipped into
+        prefix_caching = prefix_caching and num_state_slots == 0
         self.native = rt.KVCacheManager(num_blocks, block_size, prefix_caching)
         self.block_size = block_size
         self.num_blocks = num_blocks
         self.prefix_caching = prefix_caching
         self._committed = {}   # seq_id -> full blocks already hashed
+        self.slots = StateSlots(num_state_slots) if num_state_slots > 0 else None
 
     @staticmethod
     def _toks(seq: Sequence) -> np.ndarray:
@@ -29,7 +67,14 @@ class BlockManager:
                                            getattr(seq, "cache_salt", 0) or 0)
 
     def ensure(self, seq: Sequence, num_tokens: int) -> bool:
+        """Blocks for the sequence's first ``num_tokens`` tokens and, for models with recurrent
+        state, its state slot (kept until ``free``)."""
+        if self.slots is not None and self.slots.acquire(seq.seq_id) < 0:
+            return False
         return self.native.ensure(seq.seq_id, num_tokens)
+
+    def state_slot(self, seq: Sequence) -> int:
+        return self.slots.slot_of(seq.seq_id) if self.slots is not None else -1
 
     def commit(self, seq: Sequence) -> None:
         if not self.prefix_caching:
@@ -43,6 +88,8 @@ class BlockManager:
 
     def free(self, seq: Sequence) -> None:
         self.native.free(seq.seq_id)
+        if self.slots is not None:
+            self.slots.release(seq.seq_id)
         self._committed.pop(seq.seq_id, None)
 
     def block_table(self, seq: Sequence):

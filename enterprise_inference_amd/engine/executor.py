@@ -112,6 +112,8 @@ def swap_enabled(runner: ModelRunner) -> bool:
     """Swapping KV into host memory only pays off from a GPU: a CPU engine's KV already lives
     in host RAM (vLLM's CPU backend has no swap space either), so it keeps recompute
     preemption -- EIA_CPU_SWAP=1 turns it on for the CPU tests of the swap machinery."""
+    if getattr(runner, "kv_buf", None) is None:
+        return False      # model-defined cache layout (latent rows, state slots): recompute
     return runner.is_gpu or os.environ.get("EIA_CPU_SWAP", "0") not in ("0", "", "false")
 
 

@@ -56,6 +56,7 @@ class StepOutput:
 _TOKEN_WAIT = __import__("os").environ.get("EIA_TOKEN_WAIT", "event")
 
 _O_NAMES = ("ids", "pos", "slot", "src", "dbt", "dlen", "pbt", "plen", "cu", "work", "lidx")
+_O_STATE = ("sslot", "scu")   # recurrent-state models: per-sequence slots and row offsets
 _PLAN_MAGIC = 0x45504C31      # "EPL1"
 _HDR_WORDS = 32
 
@@ -89,6 +90,8 @@ class StepPlan:
             h[16 + i] = self.o.get(n, -1)
         h[27] = int(bool(self.sharded))
         h[28] = 0 if self.swap is None else len(self.swap)
+        for i, n in enumerate(_O_STATE):
+            h[29 + i] = self.o.get(n, -1)
         return h
 
     @classmethod
@@ -101,6 +104,7 @@ class StepPlan:
                 n_sample=int(h[13]), unfiltered=bool(h[14]), sharded=bool(h[27]))
         if p.kind == "eager":
             p.o = {n: int(h[16 + i]) for i, n in enumerate(_O_NAMES)}
+            p.o.update({n: int(h[29 + i]) for i, n in enumerate(_O_STATE) if int(h[29 + i]) >= 0})
         p.swap = int(h[28])          # word count; load_message replaces it with the words
         return p, int(h[15])
 
@@ -144,6 +148,11 @@ class ModelRunner:
             _native.kernels()         # fail loudly now if the HIP library is unusable
             from ..ops import gemm as _gemm_ops
             _gemm_ops.enable_prefill_tuning()
+            if cfg.dtype == torch.float32:
+                # fp32 serving means true fp32 products: no reduced-precision matrix mode
+                torch.backends.cuda.matmul.allow_tf32 = False
+                torch.backends.cudnn.allow_tf32 = False
+                torch.set_float32_matmul_precision("highest")
         elif "OMP_NUM_THREADS" not in os.environ and hasattr(os, "sched_getaffinity"):
             # CPU serving pod: one intra-op thread per core of the pod's cpuset (the NRI
             # balloon), not per core of the host
@@ -179,6 +188,12 @@ class ModelRunner:
         self.hidden_size = m.hidden_size
         self.head_dim = m.head_dim
         self.num_kv_heads = self.model.kv_heads_per_rank()
+        # models that lay out their own caches (latent rows, recurrent state slots) allocate
+        # them through allocate_cache(); the block tables, slots and batching stay the same
+        self.custom_cache = hasattr(self.model, "allocate_cache")
+        self.num_state_slots = cfg.cache.num_state_slots if getattr(
+            self.model, "needs_state_slots", False) else 0
+        self.kv_buf = None
         self.block_size = cfg.cache.block_size
         self.max_num_seqs = cfg.scheduler.max_num_seqs
         self.max_tokens = cfg.scheduler.max_num_batched_tokens
@@ -206,8 +221,7 @@ class ModelRunner:
     # ------------------------------------------------------------------ buffers
     def _alloc_staging(self) -> None:
         T, S, mb = self.max_tokens, self.max_num_seqs, self.maxb
-        qb = attn_ops.prefill_query_block(self.num_heads, self.num_kv_heads, self.head_dim,
-                                          block_size=self.block_size)
+        qb = self._query_block()
         self.max_work = T // qb + S + 1
         pin = self.is_gpu
         # graph (decode) header, fixed offsets:
@@ -217,7 +231,8 @@ class ModelRunner:
         self.hdr_len = 5 * S + 4
         self.src_off = 4 * S + 4
         # eager region: packed per step
-        self.e_size = 3 * T + 2 * S * mb + 4 * S + 1 + 2 * self.max_work + S + 64
+        self.e_size = 3 * T + 2 * S * mb + 4 * S + 1 + 2 * self.max_work + S + 64 + \
+            max(S, T) + 2 * S + 1
         # Host staging is double-buffered: with overlapped scheduling step k+1 is prepared
         # while step k's H2D copies may still be queued behind step k-1 on the stream.
         self._pin = [self._pinned_set(pin) for _ in range(2)]
@@ -246,6 +261,14 @@ class ModelRunner:
         # arrival counters of the in-kernel partition merge (kernels leave them zeroed)
         self.part_cnt = torch.zeros(S * self.num_heads, dtype=torch.int32,
                                     device=dev) if self.is_gpu else None
+
+    def _query_block(self) -> int:
+        """Queries per prefill work item of this model's attention kernel."""
+        hook = getattr(self.model, "prefill_query_block", None)
+        if hook is not None:
+            return int(hook(self.block_size))
+        return attn_ops.prefill_query_block(self.num_heads, self.num_kv_heads, self.head_dim,
+                                            block_size=self.block_size)
 
     def _sampling_views(self, buf: torch.Tensor):
         S = self.max_num_seqs
@@ -302,6 +325,8 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ KV cache
     def kv_block_bytes(self) -> int:
+        if self.custom_cache:
+            return int(self.model.cache_block_bytes(self.block_size, self.cfg.cache.cache_dtype))
         e = torch.tensor([], dtype=self.cfg.cache.cache_dtype).element_size()
         return self.num_local_layers * 2 * self.num_kv_heads * self.block_size * self.head_dim * e
 
@@ -323,6 +348,8 @@ class ModelRunner:
         reserve = 2 << 30                                     # graphs + logits + slack
         budget = total * cc.gpu_memory_utilization - peak - reserve
         budget = min(budget, free - (1 << 30) - (peak - used_now))
+        if self.num_state_slots:
+            budget -= self.num_state_slots * self.model.state_slot_bytes()
         nb = int(budget // per)
         if nb <= 0:
             raise RuntimeError("not enough GPU memory for the KV cache; lower max_num_batched_tokens"
@@ -346,14 +373,26 @@ class ModelRunner:
         cu = torch.tensor([0] + list(np.cumsum(qls)), dtype=torch.int32, device=self.device)
         lens = torch.tensor(qls, dtype=torch.int32, device=self.device)
         bt = torch.zeros(nseq, max(1, self.maxb), dtype=torch.int32, device=self.device)
-        qb = attn_ops.prefill_query_block(self.num_heads, self.num_kv_heads, self.head_dim,
-                                          block_size=self.block_size)
-        work = attn_ops.build_prefill_work(qls, qb)
+        work = attn_ops.build_prefill_work(qls, self._query_block())
         md = attn_ops.AttentionMetadata(
             num_decode=0, num_prefill_tokens=n, slot_mapping=slots, positions=pos,
             prefill_block_tables=bt, prefill_seq_lens=torch.ones_like(lens),
             prefill_cu_q=cu, prefill_work=torch.tensor(work, dtype=torch.int32, device=self.device),
             prefill_n_work=len(work) // 2, causal=False)
+        if self.custom_cache:
+            # scratch caches of one block / one slot; every sequence at position 0 of slot 0
+            md.positions = pos = torch.cat([torch.arange(q, dtype=torch.int32, device=self.device)
+                                            % self.block_size for q in qls])
+            md.num_seqs, md.seq_cu = nseq, cu
+            md.seq_slots = torch.zeros(nseq, dtype=torch.int32, device=self.device)
+            with torch.no_grad():
+                caches = self.model.allocate_cache(1, self.block_size, 1,
+                                                   self.cfg.cache.cache_dtype, self.device)
+                h = self._forward(ids, md, caches)
+                idx = torch.arange(min(n, self.max_num_seqs), device=self.device)
+                self.model.compute_logits(h[idx])
+            del h, caches
+            return
         with torch.no_grad():
             inter = None
             if self.pp > 1 and not pstate.is_first_stage():
@@ -368,6 +407,12 @@ class ModelRunner:
     def allocate_kv_cache(self, num_blocks: Optional[int] = None) -> int:
         nb = num_blocks or self.determine_num_blocks()
         self.num_blocks = nb
+        if self.custom_cache:
+            self.kv_caches = self.model.allocate_cache(nb, self.block_size, self.num_state_slots,
+                                                       self.cfg.cache.cache_dtype, self.device)
+            logger.info("cache: %d blocks x %d tokens, %d state slots (model-defined layout)",
+                        nb, self.block_size, self.num_state_slots)
+            return nb
         Hkv, bs, D = self.num_kv_heads, self.block_size, self.head_dim
         per_layer = nb * Hkv * bs * D
         # zero-filled: never-written slots must stay finite (masked P=0 times V)
@@ -522,7 +567,8 @@ class ModelRunner:
         """Vocab shards -> full fp32 logits (a collective: every TP rank calls it)."""
         return self.model.lm_head.gather(local).float()
 
-    def _prepare_eager(self, bm: BlockManager, out: SchedulerOutput) -> dict:
+    def _prepare_eager(self, bm: BlockManager, out: SchedulerOutput,
+                       logit_rows: Optional[List[int]] = None) -> dict:
         """Pack the step's metadata into the eager staging buffer; returns the plan."""
         buf = self.e_buf.numpy()
         base = self.e_buf.data_ptr()
@@ -571,9 +617,7 @@ class ModelRunner:
                             base + 4 * o["plen"], T - nd)
             buf[o["cu"]] = 0
             buf[o["cu"] + 1:o["cu"] + 1 + npf] = np.cumsum(qlens)
-        qb = attn_ops.prefill_query_block(self.num_heads, self.num_kv_heads, self.head_dim,
-                                          block_size=self.block_size)
-        work = attn_ops.build_prefill_work(qlens, qb)
+        work = attn_ops.build_prefill_work(qlens, self._query_block())
         take("work", len(work))
         if work:
             buf[o["work"]:o["work"] + len(work)] = work
@@ -583,9 +627,19 @@ class ModelRunner:
             acc += it.num_tokens
             if it.samples:
                 sample_rows.append(acc - 1)
+        if logit_rows is not None:       # the caller names the rows whose logits it wants
+            sample_rows = list(logit_rows)
         take("lidx", len(sample_rows))
         if sample_rows:
             buf[o["lidx"]:o["lidx"] + len(sample_rows)] = sample_rows
+        if self.num_state_slots:
+            # sequences in batch order with their state slots and row ranges
+            take("sslot", nd + npf)
+            take("scu", nd + npf + 1)
+            seqs = [d.seq for d in out.decodes] + [d.seq for d in out.prefills]
+            buf[o["sslot"]:o["sslot"] + nd + npf] = [bm.state_slot(q) for q in seqs]
+            buf[o["scu"]] = 0
+            buf[o["scu"] + 1:o["scu"] + 1 + nd + npf] = np.cumsum([1] * nd + qlens)
         max_len = max([it.start + it.num_tokens for it in out.decodes], default=1)
         P = self._decode_partitions(nd, max_len) if nd else 1
         return StepPlan("eager", T=T, nd=nd, npf=npf, mb_d=mb_d, mb_p=mb_p, o=o,
@@ -606,6 +660,11 @@ class ModelRunner:
             prefill_cu_q=d[o["cu"]:o["cu"] + npf + 1] if npf else None,
             prefill_work=d[o["work"]:o["work"] + 2 * nw] if npf else None,
             prefill_n_work=nw)
+        if "sslot" in o:
+            ns = nd + npf
+            md.num_seqs = ns
+            md.seq_slots = d[o["sslot"]:o["sslot"] + ns]
+            md.seq_cu = d[o["scu"]:o["scu"] + ns + 1]
         lidx = d[o["lidx"]:o["lidx"] + plan["n_lidx"]].long()
         ids = d[o["ids"]:o["ids"] + T]
         if plan.get("src"):
@@ -893,6 +952,22 @@ class ModelRunner:
             self.finish_step()
 
     @torch.no_grad()
+    def step_logits(self, bm: BlockManager, out: SchedulerOutput,
+                    rows: List[int]) -> Optional[torch.Tensor]:
+        """Run one step without sampling and return the fp32 logits of the given batch rows
+        (rows index the step's token layout [decode rows | prefill chunks]); the same staging,
+        forward and cache writes as a sampled step."""
+        self._flip_staging()
+        plan = self._prepare_eager(bm, out, logit_rows=rows)
+        plan.mm = self._mm_rows(out)
+        try:
+            logits = self.run(plan)
+            self.last_rows = {}
+            return None if logits is None else logits.float()
+        finally:
+            self.finish_step()
+
+    @torch.no_grad()
     def execute(self, bm: BlockManager, out: SchedulerOutput) -> StepOutput:
         return self.launch(bm, out, overlap=False).result()
 
@@ -910,7 +985,8 @@ class ModelRunner:
     # ------------------------------------------------------------------ graphs
     @torch.no_grad()
     def capture_graphs(self, buckets: Optional[List[int]] = None) -> float:
-        if not self.is_gpu or self.cfg.enforce_eager or self.pp > 1:
+        if not self.is_gpu or self.cfg.enforce_eager or self.pp > 1 or \
+                not getattr(self.model, "supports_graphs", True):
             return 0.0
         t0 = time.time()
         buckets = buckets or graph_buckets(self.max_num_seqs, self.cfg.scheduler.decode_bs_bucket_step)

@@ -64,7 +64,8 @@ class Scheduler:
         self.cfg = sched
         self.cache_cfg = cache
         self.bm = block_manager or BlockManager(num_blocks, cache.block_size,
-                                                cache.enable_prefix_caching)
+                                                cache.enable_prefix_caching,
+                                                getattr(cache, "num_state_slots", 0))
         self.waiting: Deque[Sequence] = collections.deque()
         self.running: List[Sequence] = []
         self.swapped: Deque[Sequence] = collections.deque()
@@ -228,6 +229,35 @@ class Scheduler:
         total = sum(s.num_tokens for s in decodes) + sum(s.num_tokens for s in prefills)
         swap_out, self._swap_out = self._swap_out, []
         return SchedulerOutput(decodes, prefills, preempted, total, swap_out, swap_in)
+
+    def plan_given(self, chunks: List[Tuple[Sequence, int]]) -> SchedulerOutput:
+        """A step whose composition the caller dictates (replaying a recorded schedule): for each
+        (sequence, n) the next ``n`` uncomputed tokens, admitted on first sight.  Same block and
+        state-slot bookkeeping as ``schedule``; nothing is preempted -- a chunk that does not
+        fit raises.  A single token after the first is a decode row, anything else a prefill
+        chunk; follow with ``update_after_step``."""
+        decodes: List[ScheduledSeq] = []
+        prefills: List[ScheduledSeq] = []
+        for seq, n in chunks:
+            if seq.status != SeqStatus.RUNNING:
+                if len(self.running) >= self.cfg.max_num_seqs:
+                    raise RuntimeError("plan_given: more live sequences than max_num_seqs")
+                try:
+                    self.waiting.remove(seq)
+                except ValueError:
+                    pass
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+            start = seq.num_computed_tokens
+            if n < 1 or start + n > seq.num_tokens:
+                raise ValueError("plan_given: chunk outside the sequence's known tokens")
+            if not self.bm.ensure(seq, start + n):
+                raise RuntimeError("plan_given: out of cache blocks or state slots")
+            (decodes if (n == 1 and start > 0) else prefills).append(ScheduledSeq(seq, start, n))
+        total = sum(c[1] for c in chunks)
+        if total > self.cfg.max_num_batched_tokens:
+            raise RuntimeError("plan_given: step exceeds max_num_batched_tokens")
+        return SchedulerOutput(decodes, prefills, [], total)
 
     def update_after_step(self, out: SchedulerOutput) -> None:
         """Advance computed-token counters and register full blocks for prefix reuse."""

@@ -17,6 +17,7 @@ _REGISTRY: Dict[str, str] = {
     "Llama4ForConditionalGeneration": "mixtral:Llama4ForCausalLM",
     "Llama4ForCausalLM": "mixtral:Llama4ForCausalLM",
     "OPTForCausalLM": "opt:OPTForCausalLM",
+    "Sekolorn": "sekolorn:SekolornForCausalLM",
     "BertModel": "bert:BertEmbeddingModel",
     "XLMRobertaModel": "bert:BertEmbeddingModel",
     "XLMRobertaForSequenceClassification": "bert:CrossEncoderModel",

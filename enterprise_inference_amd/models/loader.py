@@ -60,7 +60,11 @@ def build_model(cfg: EngineConfig, device: torch.device) -> nn.Module:
                          "must be requested explicitly)")
     if fmt == "dummy":
         logger.info("random-init weights (load_format=%s, no checkpoint)", fmt)
-        init_random_(model, seed=cfg.seed)
+        own = getattr(model, "init_random", None)     # designs with non-standard parameter names
+        if own is not None:
+            own(cfg.seed)
+        else:
+            init_random_(model, seed=cfg.seed)
         post = getattr(model, "post_load", None)
         if post:
             post()
@@ -87,6 +91,9 @@ def resolve_model_config(model: str, hf_overrides: Optional[dict] = None) -> Mod
     if os.path.isdir(model) and os.path.exists(os.path.join(model, "config.json")):
         with open(os.path.join(model, "config.json")) as f:
             d = json.load(f)
+        if isinstance(d.get("architecture"), str) and isinstance(d.get("layers"), list) \
+                and not hf_overrides:
+            return ModelConfig.from_pretrained(model)     # also reads tensor shapes
     else:
         d = get_preset(model)
     if hf_overrides:

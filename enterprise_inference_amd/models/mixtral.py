@@ -197,6 +197,54 @@ class MixtralMoE(nn.Module):
         return _deferred_reduce(out)
 
 
+class UngatedMLP(nn.Module):
+    """W_down act(W_up x) without a gate branch (act: squared ReLU)."""
+
+    def __init__(self, hidden: int, inter: int, dtype, device):
+        super().__init__()
+        self.up = ReplicatedLinear(hidden, inter, dtype=dtype, device=device)
+        self.down = ReplicatedLinear(inter, hidden, dtype=dtype, device=device)
+
+    def forward(self, x):
+        from ..ops import activation
+        return self.down(activation.relu2(self.up(x)))
+
+
+class GroupRoutedMoE(nn.Module):
+    """Ungated experts behind a group-limited sigmoid router (ops/moe.py route_grouped +
+    ungated_moe), plus an optional always-on shared expert.  One rank."""
+
+    def __init__(self, hidden: int, inter: int, num_experts: int, top_k: int, num_groups: int,
+                 keep_groups: int, route_scale: float, shared_inter: int = 0,
+                 dtype=torch.bfloat16, device=None):
+        super().__init__()
+        if state.tp_size() != 1:
+            raise NotImplementedError("GroupRoutedMoE runs on one rank")
+        if num_experts % num_groups or not (1 <= keep_groups <= num_groups) or \
+                top_k > keep_groups * (num_experts // num_groups):
+            raise ValueError("router groups do not fit the expert count / top-k")
+        self.E, self.k, self.groups, self.keep = num_experts, top_k, num_groups, keep_groups
+        self.route_scale = float(route_scale)
+        self.router = _param((num_experts, hidden), dtype, device)
+        self.w_up = _param((num_experts, inter, hidden), dtype, device)
+        self.w_down = _param((num_experts, hidden, inter), dtype, device)
+        self.router.weight_loader = lambda p, t, sid=None: p.data.copy_(t)
+        self.w_up.weight_loader = self.w_down.weight_loader = \
+            lambda p, t, sid=None: p.data[sid].copy_(t)
+        self.shared = UngatedMLP(hidden, shared_inter, dtype, device) if shared_inter else None
+
+    def forward(self, x, md=None):
+        row_len = None
+        if md is not None and md.num_prefill_tokens == 0 and md.decode_seq_lens is not None:
+            row_len = md.decode_seq_lens          # bucket-padding rows route nowhere
+        tw, ids = moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
+                                        self.route_scale, row_len)
+        out = moe_ops.ungated_moe(x, self.w_up, self.w_down, tw, ids, "relu2")
+        if self.shared is not None:
+            out = out + self.shared(x)
+        return out
+
+
 class MixtralForCausalLM(LlamaForCausalLM):
     def __init__(self, cfg: ModelConfig, dtype=torch.bfloat16, device=None):
         super().__init__(cfg, dtype, device, layer_factory=lambda i: LlamaDecoderLayer(

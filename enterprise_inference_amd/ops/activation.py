@@ -41,3 +41,14 @@ def activation(x: torch.Tensor, act: str) -> torch.Tensor:
     out = torch.empty_like(x)
     check(lib().eia_act(ptr(out), ptr(x), x.numel(), kind, stream(x)), "activation")
     return out
+
+
+def relu2(x: torch.Tensor) -> torch.Tensor:
+    """Squared ReLU, max(x, 0)^2 (bf16 or fp32)."""
+    if not (use_hip(x) and x.is_contiguous() and x.dtype in (torch.bfloat16, torch.float32)):
+        r = torch.relu(x.float())
+        return (r * r).to(x.dtype)
+    out = torch.empty_like(x)
+    check(lib().eia_relu2(ptr(out), ptr(x), x.numel(), 1 if x.dtype == torch.bfloat16 else 0,
+                          stream(x)), "relu2")
+    return out

@@ -157,6 +157,11 @@ class AttentionMetadata:
     # multimodal: batch rows whose token embedding is replaced (image placeholders)
     mm_rows: Optional[torch.Tensor] = None               # [n] int64
     mm_embeds: Optional[torch.Tensor] = None             # [n, hidden]
+    # recurrent-state models: the step's sequences in batch order (decode rows, then prefill
+    # chunks), their state slots and row ranges (None: one row per sequence, a decode step)
+    num_seqs: int = 0
+    seq_slots: Optional[torch.Tensor] = None             # [num_seqs] int32 (< 0: padding row)
+    seq_cu: Optional[torch.Tensor] = None                # [num_seqs + 1] int32
 
     @property
     def num_tokens(self) -> int:

@@ -325,3 +325,87 @@ def _fused_moe_per_expert(x, w13, w2, topk_w, topk_ids, e_lo, act):
         y = F.linear(h, w2[e])
         out.index_add_(0, tok, y.float() * topk_w[tok, slot, None])
     return out.to(x.dtype)
+
+
+def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: int,
+                  keep_groups: int, route_scale: float,
+                  row_len: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Group-limited sigmoid routing (moe.hip route_grouped_kernel): fp32 logits x W_r^T,
+    scores = sigmoid; experts form ``num_groups`` equal groups of neighbours, a group scores the
+    sum of its two largest scores, only the ``keep_groups`` best groups are eligible, the ``k``
+    largest eligible scores win and weigh score * route_scale (not renormalised; ties to the
+    lower index).  -> (weights fp32 [T, k], expert ids int32 [T, k])."""
+    T, H = x.shape
+    E = router_w.shape[0]
+    if not use_hip(x):
+        s = torch.sigmoid(x.float() @ router_w.float().t())
+        per = E // num_groups
+        gs = s.view(T, num_groups, per).topk(min(2, per), -1).values.sum(-1)
+        # stable descending order: ties keep the lower index
+        gi = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep_groups]
+        ok = torch.zeros(T, num_groups, dtype=torch.bool)
+        ok.scatter_(1, gi, True)
+        masked = torch.where(ok[:, :, None].expand(T, num_groups, per).reshape(T, E), s,
+                             torch.full_like(s, -1.0))
+        order = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :k]
+        return s.gather(1, order) * route_scale, order.to(torch.int32)
+    require(x.stride(1) == 1 and router_w.is_contiguous() and router_w.dtype == x.dtype and
+            x.dtype in (torch.bfloat16, torch.float32), "route_grouped: layout")
+    w = torch.empty(T, k, dtype=torch.float32, device=x.device)
+    ids = torch.empty(T, k, dtype=torch.int32, device=x.device)
+    check(lib().eia_moe_route_grouped(ptr(x), x.stride(0), ptr(router_w), H, T, E, k, num_groups,
+                                      keep_groups, float(route_scale), ptr(w), ptr(ids),
+                                      ptr(row_len), 1 if x.dtype == torch.bfloat16 else 0,
+                                      stream(x)), "moe_route_grouped")
+    return w, ids
+
+
+def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_w: torch.Tensor,
+                topk_ids: torch.Tensor, act: str = "relu2") -> torch.Tensor:
+    """Experts without a gate branch: y = sum_k w_k * W_down[e_k] act(W_up[e_k] x).
+    x [T, H]; w_up [E, I, H]; w_down [E, H, I] -> [T, H].  Rows are sorted by expert on the
+    device (moe.hip align), the E+1 offsets are read back once, and each expert runs one library
+    GEMM pair on its contiguous slice; one activation launch covers all slices.  An id >= E
+    routes nowhere."""
+    from . import activation
+    T, H = x.shape
+    E, I, _ = w_up.shape
+    k = topk_ids.shape[1]
+    n = T * k
+    if not use_hip(x):
+        out = torch.zeros(T, H, dtype=torch.float32)
+        xf = x.float()
+        for e in range(E):
+            tok, slot = (topk_ids.long() == e).nonzero(as_tuple=True)
+            if tok.numel() == 0:
+                continue
+            hmid = activation.relu2(xf[tok] @ w_up[e].float().t()) if act == "relu2" else \
+                activation.activation(xf[tok] @ w_up[e].float().t(), act)
+            out.index_add_(0, tok, (hmid @ w_down[e].float().t()) * topk_w[tok, slot, None])
+        return out.to(x.dtype)
+    if act != "relu2":
+        raise NotImplementedError(f"ungated_moe: activation {act}")
+    dev = x.device
+    st = stream(x)
+    offs, row_idx, inv = _align(topk_ids, E, 0, E, n, dev, st)
+    bounds = offs.tolist()                      # the one host synchronisation of this layer
+    xs = x.index_select(0, row_idx[:bounds[E]].long())
+    h1 = torch.empty(max(1, n), I, dtype=x.dtype, device=dev)
+    for e in range(E):
+        a, b = bounds[e], bounds[e + 1]
+        if a < b:
+            torch.matmul(xs[a:b], w_up[e].t(), out=h1[a:b])
+    h1 = activation.relu2(h1)
+    h2 = torch.zeros(max(1, n), H, dtype=x.dtype, device=dev) if bounds[E] < n else \
+        torch.empty(max(1, n), H, dtype=x.dtype, device=dev)
+    for e in range(E):
+        a, b = bounds[e], bounds[e + 1]
+        if a < b:
+            torch.matmul(h1[a:b], w_down[e].t(), out=h2[a:b])
+    if x.dtype == torch.bfloat16 and H % 8 == 0:
+        out = torch.empty(T, H, dtype=x.dtype, device=dev)
+        check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
+                                    ptr(out), out.stride(0), st), "moe_combine")
+        return out
+    rows = h2.index_select(0, inv[:n].long().clamp_(0, max(0, n - 1))).view(T, k, H)
+    return (rows.float() * topk_w[:, :, None]).sum(1).to(x.dtype)

@@ -64,3 +64,39 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tenso
     check(lib().eia_layer_norm(ptr(o), ptr(x2), ptr(r2), ptr(weight), ptr(bias), float(eps), T, H,
                                stream(x)), "layer_norm")
     return o.view(x.shape)
+
+
+def post_norm_residual(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor,
+                       copy: bool = True) -> Optional[torch.Tensor]:
+    """Sublayer-output norm with an fp32 residual stream: x += layernorm(y) * weight in place
+    (no bias, variance = mean of squared deviations, all fp32); returns the new x in y's dtype
+    for the next GEMMs (``copy``; an fp32 model reads x itself)."""
+    if not use_hip(y, x):
+        yf = y.float()
+        d = yf - yf.mean(-1, keepdim=True)
+        x += d / torch.sqrt((d * d).mean(-1, keepdim=True) + eps) * weight.float()
+        return x.to(y.dtype) if copy and y.dtype != torch.float32 else (x if copy else None)
+    require(x.dtype == torch.float32 and x.is_contiguous() and y.stride(-1) == 1 and
+            y.shape == x.shape and weight.dtype == y.dtype, "post_norm_residual: layout")
+    bf = y.dtype == torch.bfloat16
+    require(bf or y.dtype == torch.float32, "post_norm_residual: bf16 or fp32")
+    T, W = x.shape
+    xb = torch.empty(T, W, dtype=y.dtype, device=y.device) if (copy and bf) else None
+    check(lib().eia_ln_residual(ptr(y), y.stride(0), ptr(weight), ptr(x), ptr(xb),
+                                W, float(eps), T, W, 1 if bf else 0, stream(y)), "ln_residual")
+    return xb if bf else (x if copy else None)
+
+
+def layer_norm_f32(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """layernorm(x fp32 [T, W]) * weight (no bias) -> [T, W] in the weight's dtype."""
+    if not use_hip(x):
+        d = x - x.mean(-1, keepdim=True)
+        return (d / torch.sqrt((d * d).mean(-1, keepdim=True) + eps) * weight.float()).to(weight.dtype)
+    require(x.dtype == torch.float32 and x.stride(-1) == 1, "layer_norm_f32: fp32 rows")
+    bf = weight.dtype == torch.bfloat16
+    require(bf or weight.dtype == torch.float32, "layer_norm_f32: bf16 or fp32 weight")
+    T, W = x.shape
+    out = torch.empty(T, W, dtype=weight.dtype, device=x.device)
+    check(lib().eia_ln_f32in(ptr(x), x.stride(0), ptr(weight), ptr(out), W, float(eps), T, W,
+                             1 if bf else 0, stream(x)), "ln_f32in")
+    return out
