@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 
 from . import reference as ref
-from ._dispatch import check, lib, ptr, stream, use_hip
+from ._dispatch import check, lib, ptr, require, stream, use_hip
 
 SCORING = {"softmax": 0, "sigmoid": 1}
 
