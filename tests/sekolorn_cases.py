@@ -1,0 +1,368 @@
+"""Sekolorn test bodies, parametrised by device and dtype: the CPU file runs them on the
+framework's PyTorch ops in fp32, the GPU file on the HIP kernels in fp32 and bf16."""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+import sekolorn_common as C
+from oracles import sekolorn_oracle as O
+
+
+def tol(dtype):
+    return 2e-4 if dtype == torch.float32 else 6e-2
+
+
+def _tokens(n, vocab, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def _weights(cfg, dtype, seed=0):
+    return C.random_weights(cfg, seed, torch.bfloat16 if dtype == torch.bfloat16 else torch.float32)
+
+
+# ------------------------------------------------------------------ mechanisms alone
+def case_post_norm(device, dtype):
+    from enterprise_inference_amd.ops import norm
+    g = torch.Generator().manual_seed(1)
+    for W in (40, 64, 257):
+        y = torch.randn(5, W, generator=g) * 3 + 1.5
+        w = torch.randn(W, generator=g)
+        x = torch.randn(5, W, generator=g)
+        want = x.double() + O.layer_norm_nobias(y.to(dtype).double(), w.to(dtype).double(), 1e-5)
+        xd = x.clone().to(device)
+        xb = norm.post_norm_residual(y.to(dtype).to(device), w.to(dtype).to(device), 1e-5, xd)
+        assert torch.allclose(xd.cpu().double(), want, atol=1e-5, rtol=1e-5)
+        assert torch.allclose(xb.float().cpu(), xd.cpu().to(dtype).float())
+        out = norm.layer_norm_f32(xd, w.to(dtype).to(device), 1e-5)
+        ref = O.layer_norm_nobias(xd.cpu().double(), w.to(dtype).double(), 1e-5)
+        assert torch.allclose(out.float().cpu().double(), ref, atol=tol(dtype), rtol=tol(dtype))
+
+
+def case_route(device, dtype):
+    from enterprise_inference_amd.ops import moe
+    g = torch.Generator().manual_seed(2)
+    for E, k, ng, keep in ((6, 2, 3, 2), (8, 3, 2, 1), (4, 2, 4, 3), (16, 3, 4, 3), (5, 1, 1, 1)):
+        H = 24
+        x = torch.randn(9, H, generator=g).to(dtype)
+        wr = (torch.randn(E, H, generator=g) * 0.7).to(dtype)
+        r = {"experts": E, "top": k, "scale": 1.3, "groups": {"count": ng, "keep": keep}}
+        tw, ids = moe.route_grouped(x.to(device), wr.to(device), k, ng, keep, 1.3)
+        for t in range(9):
+            want_ids, want_w = O.route(x[t].double(), {"router": wr.double()}, "", r)
+            assert ids[t].tolist() == want_ids, (E, k, ng, keep, t)
+            assert torch.allclose(tw[t].cpu().double(), torch.tensor(want_w, dtype=torch.float64),
+                                  atol=1e-5)
+
+
+def case_route_group_limit(device, dtype):
+    """The largest single score sits in a group whose second score is tiny: the group loses, so
+    that expert must NOT be chosen although it tops the plain ranking."""
+    from enterprise_inference_amd.ops import moe
+    E, H = 8, 8
+    wr = torch.zeros(E, H)
+    x = torch.zeros(1, H)
+    x[0, 0] = 1.0
+    # group 0 = experts 0..3: one huge, three tiny; group 1 = experts 4..7: all fairly large
+    wr[:, 0] = torch.tensor([4.0, -6.0, -6.0, -6.0, 2.0, 1.9, 1.8, 1.7])
+    tw, ids = moe.route_grouped(x.to(dtype).to(device), wr.to(dtype).to(device), 2, 2, 1, 1.0)
+    assert ids[0].tolist() == [4, 5]
+    assert abs(float(tw[0, 0]) - 1 / (1 + math.exp(-2.0))) < 1e-5
+
+
+def case_ungated_moe(device, dtype):
+    from enterprise_inference_amd.ops import moe
+    g = torch.Generator().manual_seed(3)
+    E, I, H, T, k = 5, 12, 24, 11, 2
+    x = torch.randn(T, H, generator=g).to(dtype)
+    up = (torch.randn(E, I, H, generator=g) / H ** 0.5).to(dtype)
+    down = (torch.randn(E, H, I, generator=g) / I ** 0.5).to(dtype)
+    ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    ids[3, 1] = E                                            # routes nowhere
+    tw = torch.rand(T, k, generator=g)
+    tw[3, 1] = 0.0
+    out = moe.ungated_moe(x.to(device), up.to(device), down.to(device), tw.to(device),
+                          ids.to(device)).float().cpu()
+    for t in range(T):
+        want = torch.zeros(H, dtype=torch.float64)
+        for s in range(k):
+            e = int(ids[t, s])
+            if e < E:
+                Wt = {"up": up[e].double(), "down": down[e].double()}
+                want += float(tw[t, s]) * O.expert(x[t].double(), Wt, "")
+        assert torch.allclose(out[t].double(), want, atol=tol(dtype) * 10, rtol=tol(dtype) * 10)
+
+
+def _paged(rows_c, rows_kr, block_size, nblocks, order, dtype, device):
+    """Scatter cache rows of one sequence into a paged cache using block list ``order``."""
+    n, R = rows_c.shape
+    rd = rows_kr.shape[1]
+    cache = torch.zeros(nblocks, block_size, R + rd, dtype=dtype)
+    for p in range(n):
+        cache[order[p // block_size], p % block_size] = torch.cat([rows_c[p], rows_kr[p]]).to(dtype)
+    return cache.to(device)
+
+
+def case_latent_attention_needle(device, dtype):
+    """One far key is made to dominate one query's scores (its latent is aligned with the
+    absorbed query and scaled up), at page borders and at the first positions: a mask or a
+    block-table slip moves the output by O(1).  Decode rows and a prefill chunk in one step."""
+    from enterprise_inference_amd.ops import latent_attention as la
+    from enterprise_inference_amd.ops.attention import AttentionMetadata
+    g = torch.Generator().manual_seed(4)
+    H, R, rd, bs, n = 3, 20, 6, 16, 83
+    rot_dims, base, scale = 4, 300.0, 0.4
+    inv = la.inv_frequencies(rot_dims, base, device)
+    c = torch.randn(n, R, generator=g).to(dtype).float()
+    kr_raw = torch.randn(n, rd, generator=g)
+    kr = torch.stack([O.rotate_interleaved(kr_raw[p].double(), p, rot_dims, base)
+                      for p in range(n)]).to(dtype).float()
+    order = [5, 2, 7, 0, 3, 6]
+    cache = _paged(c, kr, bs, 8, order, dtype, device)
+    qpos = [0, 1, 15, 16, 17, 31, 32, 47, 48, 63, 64, 65, 82]       # chunk rows' positions vary
+    # one prefill chunk of consecutive positions 60..82 and three decode rows of other "sequences"
+    # sharing the same pages (their own block tables point at the same blocks)
+    chunk = list(range(60, 83))
+    dec = [0, 16, 48]
+    rows = dec + chunk
+    T = len(rows)
+    qa = torch.randn(T, H, R, generator=g)
+    qr = torch.randn(T, H, rd, generator=g)
+    needles = {}
+    for i, p in enumerate(rows):
+        tgt = [0, 15, 16, 31, 32, 63, 64, p][i % 8]
+        tgt = min(tgt, p)
+        needles[i] = tgt
+        qa[i, i % H] = c[tgt] * (6.0 / scale / float(c[tgt] @ c[tgt]))
+    qa, qr = qa.to(dtype), qr.to(dtype)
+    gate = torch.randn(T, H, generator=g).to(dtype)
+    bt = torch.tensor(order + [0, 0], dtype=torch.int32)
+    md = AttentionMetadata(
+        num_decode=len(dec), num_prefill_tokens=len(chunk),
+        slot_mapping=torch.full((T,), -1, dtype=torch.int32, device=device),
+        positions=torch.tensor(rows, dtype=torch.int32, device=device),
+        decode_block_tables=bt.repeat(len(dec), 1).to(device),
+        decode_seq_lens=torch.tensor([p + 1 for p in dec], dtype=torch.int32, device=device),
+        prefill_block_tables=bt[None].to(device),
+        prefill_seq_lens=torch.tensor([83], dtype=torch.int32, device=device),
+        prefill_cu_q=torch.tensor([0, len(chunk)], dtype=torch.int32, device=device))
+    for qb in (1, 4, 16):
+        work = la.build_work([len(chunk)], qb)
+        md.prefill_work = torch.tensor(work, dtype=torch.int32, device=device)
+        md.prefill_n_work = len(work) // 2
+        out = la.latent_attention(qa.to(device), qr.to(device), inv, rot_dims, cache, md,
+                                  gate.to(device), scale, qb).float().cpu()
+        for i, p in enumerate(rows):
+            for h in range(H):
+                q_rot = O.rotate_interleaved(qr[i, h].double(), p, rot_dims, base)
+                s = torch.tensor([(qa[i, h].double() @ c[j].double() + q_rot @ kr[j].double())
+                                  * scale for j in range(p + 1)])
+                a = torch.softmax(s, 0)
+                want = (a[:, None] * c[:p + 1].double()).sum(0) * torch.sigmoid(gate[i, h].double())
+                assert torch.allclose(out[i, h].double(), want, atol=tol(dtype) * 5,
+                                      rtol=tol(dtype) * 5), (qb, i, p, h, needles[i])
+
+
+def case_latent_prep(device, dtype):
+    from enterprise_inference_amd.ops import latent_attention as la
+    g = torch.Generator().manual_seed(5)
+    T, Q, R, rd, rot_dims, base, bs = 7, 10, 12, 6, 4, 77.0, 16
+    fused = torch.randn(T, Q + R + rd + 2, generator=g).to(dtype)
+    wq, wc = torch.randn(Q, generator=g).to(dtype), torch.randn(R, generator=g).to(dtype)
+    pos = torch.tensor([0, 1, 2, 40, 41, 15, 16], dtype=torch.int32)
+    slots = torch.tensor([3, 4, -1, 33, 34, 63, 16], dtype=torch.int32)
+    cache = torch.zeros(4, bs, R + rd, dtype=dtype, device=device)
+    inv = la.inv_frequencies(rot_dims, base, device)
+    cq = la.latent_prep(fused.to(device), 0, Q, wq.to(device), Q, R, wc.to(device), Q + R, rd,
+                        rot_dims, inv, pos.to(device), slots.to(device), cache, 1e-5)
+    flat = cache.view(-1, R + rd).float().cpu()
+    f = fused.double()
+    for t in range(T):
+        want_q = O.rms_unit(f[t, :Q], 1e-5) * wq.double()
+        assert torch.allclose(cq[t].float().cpu().double(), want_q, atol=tol(dtype), rtol=tol(dtype))
+        if slots[t] < 0:
+            continue
+        want_c = O.rms_unit(f[t, Q:Q + R], 1e-5) * wc.double()
+        want_k = O.rotate_interleaved(f[t, Q + R:Q + R + rd], int(pos[t]), rot_dims, base)
+        got = flat[int(slots[t])].double()
+        assert torch.allclose(got[:R], want_c, atol=tol(dtype), rtol=tol(dtype))
+        assert torch.allclose(got[R:], want_k, atol=tol(dtype), rtol=tol(dtype))
+    assert float(flat[5].abs().sum()) == 0.0          # the skipped row wrote nothing
+
+
+def case_wkv(device, dtype):
+    """Token shift + scan on two sequences (one continuing from a slot's state, one fresh in a
+    slot that holds stale values) against the per-token oracle."""
+    from enterprise_inference_amd.ops import wkv
+    for H, D, Wd in ((3, 16, 40), (2, 72, 48), (1, 64, 64)):
+        g = torch.Generator().manual_seed(6 + D)
+        m = {"heads": H, "dim": D}
+        HD = H * D
+        Wt = {"mu." + s: torch.rand(Wd, generator=g) for s in "rkvgw"}
+        for s in "rkvg":
+            Wt[s] = torch.randn(HD, Wd, generator=g) / Wd ** 0.5
+        Wt.update({"w1": torch.randn(5, Wd, generator=g) / Wd ** 0.5,
+                   "w2": torch.randn(HD, 5, generator=g), "w0": torch.randn(HD, generator=g) - 1,
+                   "u": torch.randn(H, D, generator=g) * 0.5,
+                   "norm": 1 + 0.2 * torch.randn(HD, generator=g),
+                   "o": torch.eye(HD)})
+        Wt = {k: v.to(dtype).double() for k, v in Wt.items()}
+        xa, xb_ = torch.randn(9, Wd, generator=g), torch.randn(4, Wd, generator=g)
+        # oracle: sequence A in two parts (5 + 4 tokens), sequence B whole
+        ya1, st = O.wkv_mixer(xa[:5].double(), Wt, "", m, 1e-5)
+        ya2, st2 = O.wkv_mixer(xa[5:].double(), Wt, "", m, 1e-5, st)
+        yb, stb = O.wkv_mixer(xb_.double(), Wt, "", m, 1e-5)
+        S = torch.randn(3, H, D, D, generator=g)              # stale values everywhere
+        prev = torch.randn(3, Wd, generator=g)
+        S[2], prev[2] = st["S"].float(), st["prev"].float()
+        S, prev = S.to(device), prev.to(device)
+        x = torch.cat([xa[5:], xb_]).to(device)              # step: A continues, B starts
+        slots = torch.tensor([2, 0], dtype=torch.int32, device=device)
+        cu = torch.tensor([0, 4, 8], dtype=torch.int32, device=device)
+        pos = torch.tensor([5, 6, 7, 8, 0, 1, 2, 3], dtype=torch.int32, device=device)
+        mu = torch.stack([Wt["mu." + s] for s in "rkvgw"]).to(dtype).to(device)
+        mix = wkv.token_shift_mix(x, mu, prev, slots, cu, 2, pos, dtype)
+        proj = [mix[i].float().cpu().double() @ Wt[s].t() for i, s in enumerate("rkvg")]
+        dec = (torch.tanh(mix[4].float().cpu().double() @ Wt["w1"].t()) @ Wt["w2"].t()).float()
+        r, k, v, gg = (p.to(dtype).to(device) for p in proj)
+        y = wkv.wkv_scan(r, k, v, gg, dec.to(device), Wt["w0"].to(dtype).to(device),
+                         Wt["u"].reshape(-1).to(dtype).to(device), Wt["norm"].to(dtype).to(device),
+                         S, prev, x, slots, cu, 2, pos, None, 1e-5, H).float().cpu().double()
+        want = torch.cat([ya2, yb])
+        scale = float(want.abs().max())
+        assert float((y - want).abs().max()) <= tol(dtype) * 20 * scale, (H, D)
+        t2 = tol(dtype) * 50
+        assert torch.allclose(S[2].cpu().double(), st2["S"], atol=t2 * float(st2["S"].abs().max()))
+        assert torch.allclose(S[0].cpu().double(), stb["S"], atol=t2 * float(stb["S"].abs().max()))
+        assert torch.allclose(prev[2].cpu(), xa[8]) and torch.allclose(prev[0].cpu(), xb_[3])
+
+
+# ------------------------------------------------------------------ whole model through the engine
+def _check(got, want, dtype, what):
+    e = C.rel_err(got, want)
+    assert e <= tol(dtype), (what, e)
+
+
+def case_schedules(device, dtype, cfg_fn=C.config_a, seed=0):
+    """Whole prompts, prompt + one-by-one decoding, portions of several sizes down to two tokens
+    and mixed batches with reuse of pages and slots all give the oracle's logits."""
+    cfg = cfg_fn()
+    W = _weights(cfg, dtype, seed)
+    V = cfg["vocab"]
+    reqs = {"a": _tokens(70, V, 11), "b": _tokens(37, V, 12), "c": _tokens(5, V, 13),
+            "d": _tokens(1, V, 14), "e": _tokens(49, V, 15)}
+    want = {k: C.oracle_logits(cfg, W, t) for k, t in reqs.items()}
+    # pool of 8 pages of 16 tokens: "a" alone needs 5, so pages must be used again
+    sess = C.make_session(cfg, W, device, dtype, max_tokens=128, block_size=16, max_live=2)
+    try:
+        # whole, each alone
+        for k, t in reqs.items():
+            got = sess.step([{"id": k, "tokens": t, "want": list(range(len(t)))}], end=[k])
+            _check(got, want[k], dtype, ("whole", k))
+        # a prompt portion, then token by token (the state and cache carry every step)
+        for k in ("a", "b"):
+            t = reqs[k]
+            n0 = len(t) - 34
+            got = [sess.step([{"id": k, "tokens": t[:n0], "want": [n0 - 1]}])]
+            for i in range(n0, len(t)):
+                got.append(sess.step([{"id": k, "tokens": [t[i]], "want": [0]}],
+                                     end=[k] if i == len(t) - 1 else []))
+            _check(torch.cat(got), want[k][n0 - 1:], dtype, ("decode", k))
+        # portions: sizes cross page borders (16) and go down to two tokens
+        t, at, got = reqs["a"], 0, []
+        for n in (2, 13, 2, 16, 1, 17, 2, 15, 2):
+            got.append(sess.step([{"id": "a", "tokens": t[at:at + n], "want": list(range(n))}],
+                                 end=["a"] if at + n == len(t) else []))
+            at += n
+        assert at == len(t)
+        _check(torch.cat(got), want["a"], dtype, "portions")
+    finally:
+        sess.close()
+    # mixed batches on 4 slots / 10 pages: unequal requests side by side, decode rows beside
+    # prompt portions, requests that pause, slots and pages freed and taken again
+    sess = C.make_session(cfg, W, device, dtype, max_tokens=160, block_size=16, max_live=4)
+    try:
+        got = {k: [] for k in reqs}
+        at = {k: 0 for k in reqs}
+
+        def run(plan, end=()):
+            entries = []
+            for k, n in plan:
+                entries.append({"id": k, "tokens": reqs[k][at[k]:at[k] + n], "want": list(range(n))})
+            out = sess.step(entries, end)
+            r = 0
+            for k, n in plan:
+                got[k].append(out[r:r + n])
+                r += n
+                at[k] += n
+        run([("d", 1), ("b", 3), ("c", 2)], end=["d"])
+        run([("b", 1), ("c", 3), ("a", 20)], end=["c"])           # c finishes: slot + page free
+        run([("a", 1), ("e", 30), ("b", 17)])                     # e takes the freed slot
+        run([("e", 1), ("b", 16), ("a", 2)], end=["b"])
+        run([("a", 47)], end=["a"])                               # e pauses
+        run([("e", 18)], end=["e"])
+        for k in reqs:
+            assert at[k] == len(reqs[k])
+            _check(torch.cat(got[k]), want[k], dtype, ("mixed", k))
+        # a second life for a finished request's name, on reused slots and pages
+        got2 = sess.step([{"id": "b", "tokens": reqs["b"], "want": list(range(len(reqs["b"])))},
+                          {"id": "c", "tokens": reqs["c"], "want": [4]}], end=["b", "c"])
+        _check(got2[:-1], want["b"], dtype, "again b")
+        _check(got2[-1:], want["c"][4:], dtype, "again c")
+        bm = sess.scheduler.bm
+        assert bm.num_free_blocks() == bm.num_blocks and bm.slots.num_free() == 4
+    finally:
+        sess.close()
+
+
+def case_long_decode(device, dtype):
+    """140 tokens decoded one by one after a 3-token prompt, over many page borders."""
+    cfg = C.config_b()
+    W = _weights(cfg, dtype, 3)
+    t = _tokens(143, cfg["vocab"], 21)
+    want = C.oracle_logits(cfg, W, t)
+    sess = C.make_session(cfg, W, device, dtype, max_tokens=160, block_size=16, max_live=1)
+    try:
+        got = [sess.step([{"id": "x", "tokens": t[:3], "want": [0, 1, 2]}])]
+        for i in range(3, len(t)):
+            got.append(sess.step([{"id": "x", "tokens": [t[i]], "want": [0]}]))
+        _check(torch.cat(got), want, dtype, "long decode")
+    finally:
+        sess.close()
+
+
+def case_generate(device, dtype):
+    """Greedy generation through LLMEngine (its scheduler, batching and sampler): every emitted
+    token is the oracle's argmax given the tokens before it, for unequal prompts in one batch."""
+    import copy
+
+    from enterprise_inference_amd.config import (CacheConfig, EngineConfig, ModelConfig,
+                                                 SchedulerConfig)
+    from enterprise_inference_amd.engine.llm_engine import LLMEngine
+    from enterprise_inference_amd.engine.sampling_params import SamplingParams
+    cfg = C.config_a()
+    W = _weights(cfg, dtype, 5)
+    ec = EngineConfig(model=ModelConfig.from_hf_dict(copy.deepcopy(cfg)), dtype=dtype, device=device,
+                      load_format="dummy",
+                      cache=CacheConfig(block_size=16, num_gpu_blocks=24),
+                      scheduler=SchedulerConfig(max_num_seqs=3, max_num_batched_tokens=32,
+                                                max_model_len=128))
+    eng = LLMEngine(ec)
+    model = eng.executor.runner.model
+    model.load_weights(W.items())
+    model.post_load()
+    prompts = [_tokens(n, cfg["vocab"], 30 + n) for n in (40, 7, 1, 19)]     # 4 prompts, 3 slots
+    outs = eng.generate(prompt_token_ids=prompts,
+                        params=SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        toks = list(o.outputs[0].token_ids)
+        assert len(toks) == 6
+        lg = C.oracle_logits(cfg, W, p + toks[:-1])
+        for i, tk in enumerate(toks):
+            row = lg[len(p) - 1 + i]
+            # the chosen token is the oracle's best, or within rounding of it
+            assert float(row.max() - row[tk]) <= (1e-3 if dtype == torch.float32 else 0.15), (i, tk)
+    eng.shutdown()

@@ -1,0 +1,46 @@
+"""Sekolorn on the MI355X path (HIP kernels; fp32 and bf16 activations) against the plain oracle
+in tests/oracles: every kernel alone, then the whole model through the engine."""
+
+import pytest
+import torch
+
+import sekolorn_cases as K
+import sekolorn_common as C
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("case", [K.case_post_norm, K.case_route, K.case_route_group_limit,
+                                  K.case_ungated_moe, K.case_latent_prep,
+                                  K.case_latent_attention_needle, K.case_wkv],
+                         ids=lambda f: f.__name__)
+def test_kernel(case, dtype):
+    case("cuda", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_schedules_config_a(dtype):
+    K.case_schedules("cuda", dtype, C.config_a)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_schedules_config_b(dtype):
+    K.case_schedules("cuda", dtype, C.config_b, seed=7)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_long_decode(dtype):
+    K.case_long_decode("cuda", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_generate_through_engine(dtype):
+    K.case_generate("cuda", dtype)
+
+
+def test_native_library_loaded():
+    from enterprise_inference_amd import _native
+    _native.kernels()
+    assert any("libeia_kernels.so" in p for p in _native.loaded_native_libraries())
