@@ -57,6 +57,20 @@ def config_b():
             ]}
 
 
+def all_experts(cfg: dict) -> dict:
+    """The same model with every expert of every group chosen.  With bf16 activations a
+    router score that nearly ties another can pick a different expert than the float64 oracle
+    does (and every later token then differs), so the bf16 whole-model comparisons take the
+    selection out; selection itself is checked in fp32 and in the routing kernel's own tests."""
+    cfg = copy.deepcopy(cfg)
+    for L in cfg["layers"]:
+        if L.get("mlp"):
+            r = L["mlp"]["router"]
+            r["top"] = r["experts"]
+            r["groups"]["keep"] = r["groups"]["count"]
+    return cfg
+
+
 def random_weights(cfg: dict, seed: int = 0, dtype=torch.float32) -> dict:
     """A checkpoint for ``cfg`` under the design's tensor names (values rounded to ``dtype``)."""
     g = torch.Generator().manual_seed(seed)

@@ -11,6 +11,11 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16]
 
 
+def _cfg(fn, dtype):
+    """fp32 runs the configuration as it is; bf16 with every expert chosen (C.all_experts)."""
+    return fn if dtype == torch.float32 else (lambda: C.all_experts(fn()))
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 @pytest.mark.parametrize("case", [K.case_post_norm, K.case_route, K.case_route_group_limit,
                                   K.case_ungated_moe, K.case_latent_prep,
@@ -22,22 +27,22 @@ def test_kernel(case, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_schedules_config_a(dtype):
-    K.case_schedules("cuda", dtype, C.config_a)
+    K.case_schedules("cuda", dtype, _cfg(C.config_a, dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_schedules_config_b(dtype):
-    K.case_schedules("cuda", dtype, C.config_b, seed=7)
+    K.case_schedules("cuda", dtype, _cfg(C.config_b, dtype), seed=7)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_long_decode(dtype):
-    K.case_long_decode("cuda", dtype)
+    K.case_long_decode("cuda", dtype, _cfg(C.config_b, dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_generate_through_engine(dtype):
-    K.case_generate("cuda", dtype)
+    K.case_generate("cuda", dtype, _cfg(C.config_a, dtype))
 
 
 def test_native_library_loaded():
