@@ -307,3 +307,264 @@ EIA_API int eia_latent_attn(const void* qa, long qa_st, long qa_sh, const void* 
   }
   EIA_LAUNCH_CHECK();
 }
+
+// --------------------------------------------------------------------------- MFMA form (bf16)
+// Flash-style kernel on v_mfma_f32_16x16x32_bf16.  A workgroup of NW waves owns NW x 16 rows
+// (row = (query, head) pair; every row reads the same keys) and walks the keys in units of 32.
+// Per unit the workgroup stages the 32 cache rows in LDS twice: row-major ("K tile", the A
+// operand of S^T = K Q^T) and transposed ("V^T tile", latent columns only, the A operand of
+// O^T = V^T P^T).  The K tile rows are stored in the order the two S^T tiles read them, so that
+// their accumulators hold, per lane, one row's scores of keys 8g..8g+7 -- exactly the B operand
+// of the second product (no shuffle, no LDS round trip for P).  Softmax weights stay fp32: P
+// is fed as a bf16 high part plus a bf16 remainder (two MFMAs), and the normaliser sums the
+// fp32 weights.  The next unit's cache rows are prefetched into registers during the products.
+template <int NKMAX, int NCMAX, int NW>
+__global__ void __launch_bounds__(NW * 64)
+latent_attn_mfma_kernel(LatentAttnArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int NT = NW * 64;
+  constexpr int PRE = (32 * NKMAX * 4 + NT - 1) / NT;      // 16-byte chunks per thread per unit
+  constexpr bool PREFETCH = PRE <= 12;                     // else the registers go to Q and O
+  const int Dk = a.R + a.rd;
+  const int nk = (Dk + 31) >> 5, Dkp = nk << 5;            // k-steps of 32
+  const int nc = (a.R + 15) >> 4;                          // latent column tiles of 16
+  const int ldk = a.ldk;                                   // K tile row stride (elements)
+  constexpr int LDV = 40;                                  // V^T tile row stride (elements)
+  bf16_t* kt = reinterpret_cast<bf16_t*>(smem);            // [32][ldk]
+  bf16_t* vt = kt + 32 * ldk;                              // [nc * 16][LDV]
+
+  int seq, row0, ntok;
+  if (a.cu_q) {
+    seq = a.work[2 * blockIdx.x];
+    const int q0 = a.work[2 * blockIdx.x + 1];
+    row0 = a.cu_q[seq] + q0;
+    ntok = min(a.QB, a.cu_q[seq + 1] - row0);
+  } else {
+    seq = blockIdx.x;
+    row0 = seq;
+    ntok = 1;
+  }
+  if (ntok <= 0 || (a.seq_lens && a.seq_lens[seq] <= 0)) return;
+  const int h0 = blockIdx.y * a.HB;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const bf16_t* cache = static_cast<const bf16_t*>(a.cache);
+  const int* bt = a.block_table + (long)seq * a.bt_stride;
+
+  // this lane's row (B operand column / accumulator column)
+  const int m = wave * 16 + c;
+  const int t = m / a.HB, h = h0 + (m - t * a.HB);
+  const bool row_ok = t < ntok && h < a.H && m < a.QB * a.HB;
+  const long row = row0 + (row_ok ? t : 0);
+  const int qpos = row_ok ? a.positions[row] : -1;
+  bf16x8 qf[NKMAX];
+  {
+    const bf16_t* qa = static_cast<const bf16_t*>(a.qa) + row * a.qa_st + (long)h * a.qa_sh;
+    const bf16_t* qr = static_cast<const bf16_t*>(a.qr) + row * a.qr_st + (long)h * a.qr_sh;
+#pragma unroll
+    for (int s = 0; s < NKMAX; ++s) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int d = s * 32 + 8 * g + e;
+        float v = 0.f;
+        if (row_ok && s < nk && d < Dk) {
+          if (d < a.R) {
+            v = bf2f(qa[d]);
+          } else {
+            const int dd = d - a.R;
+            v = bf2f(qr[dd]);
+            if (dd < a.rot_dims) {
+              const int i = dd >> 1;
+              float sn, cs;
+              sincosf((float)qpos * a.inv_freq[i], &sn, &cs);
+              const float u = bf2f(qr[2 * i]), w = bf2f(qr[2 * i + 1]);
+              v = (dd & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
+            }
+          }
+        }
+        qf[s][e] = f2bf(v);
+      }
+    }
+  }
+  f32x4 acc[NCMAX];
+#pragma unroll
+  for (int i = 0; i < NCMAX; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  float mrun = -INFINITY, lrun = 0.f;
+  const float scale_log2 = a.scale * 1.4426950408889634f;
+  const int kmax = a.positions[row0 + ntok - 1] + 1;
+  const int cpr = Dkp >> 3;                                // 16-byte chunks per (padded) key row
+  const int nchunk = 32 * cpr;
+
+  auto load_chunk = [&](int k0, int ch) {
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int j = ch / cpr, d = (ch - j * cpr) << 3;
+    const int kp = k0 + j;
+    if (kp < kmax && d < Dk) {                             // Dk % 8 == 0: whole chunk inside
+      const long slot = (long)bt[kp / a.bs] * a.bs + (kp % a.bs);
+      v = *reinterpret_cast<const bf16x8*>(cache + slot * a.cache_row + d);
+    }
+    return v;
+  };
+  // key j = 8G + i lands in K tile row 4G + i (i < 4) or 16 + 4G + i - 4
+  auto store_chunk = [&](int ch, bf16x8 v) {
+    const int j = ch / cpr, d = (ch - j * cpr) << 3;
+    const int r = ((j & 4) ? 16 : 0) + 4 * (j >> 3) + (j & 3);
+    *reinterpret_cast<bf16x8*>(kt + r * ldk + d) = v;
+  };
+  bf16x8 pre[PREFETCH ? PRE : 1];
+  auto fetch = [&](int k0) {
+    if constexpr (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < PRE; ++i) {
+        const int ch = tid + i * NT;
+        if (ch < nchunk) pre[i] = load_chunk(k0, ch);
+      }
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < kmax; k0 += 32) {
+    if constexpr (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < PRE; ++i) {
+        const int ch = tid + i * NT;
+        if (ch < nchunk) store_chunk(ch, pre[i]);
+      }
+    } else {
+      for (int ch = tid; ch < nchunk; ch += NT) store_chunk(ch, load_chunk(k0, ch));
+    }
+    __syncthreads();
+    // K tile -> V^T tile (latent columns; rows past R are zero from the padded chunks)
+    for (int ch = tid; ch < 32 * nc * 2; ch += NT) {
+      const int j = ch & 31, d = (ch >> 5) << 3;
+      const int r = ((j & 4) ? 16 : 0) + 4 * (j >> 3) + (j & 3);
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (d < a.R) v = *reinterpret_cast<const bf16x8*>(kt + r * ldk + d);   // R % 8 == 0
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(d + e) * LDV + j] = v[e];
+    }
+    __syncthreads();
+    if (k0 + 32 < kmax) fetch(k0 + 32);
+    // S^T tiles: keys (rows) x this wave's 16 rows (columns)
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < NKMAX; ++s) {
+      if (s < nk) {
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kt + c * ldk + s * 32 + 8 * g);
+        const bf16x8 kb = *reinterpret_cast<const bf16x8*>(kt + (16 + c) * ldk + s * 32 + 8 * g);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[s], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[s], s1, 0, 0, 0);
+      }
+    }
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ka = k0 + 8 * g + i, kb = ka + 4;
+      v[i] = (ka <= qpos) ? s0[i] * scale_log2 : -INFINITY;
+      v[4 + i] = (kb <= qpos) ? s1[i] * scale_log2 : -INFINITY;
+    }
+    float mloc = v[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) mloc = fmaxf(mloc, v[i]);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+    const float mnew = fmaxf(mrun, mloc);
+    const float muse = (mnew == -INFINITY) ? 0.f : mnew;
+    const float alpha = exp2f(mrun - muse);                // mrun = -inf: 0 (nothing summed yet)
+    bf16x8 ph, pl;
+    float psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float p = exp2f(v[i] - muse);
+      const bf16_t hi = f2bf(p);
+      ph[i] = hi;
+      pl[i] = f2bf(p - bf2f(hi));
+      psum += p;
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    lrun = lrun * alpha + psum;
+    mrun = mnew;
+    const bool rescale = !__all(alpha == 1.f);
+#pragma unroll
+    for (int ct = 0; ct < NCMAX; ++ct) {
+      if (ct < nc) {
+        const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (ct * 16 + c) * LDV + 8 * g);
+        f32x4 o = acc[ct];
+        if (rescale) o *= alpha;
+        o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, o, 0, 0, 0);
+        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o, 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  if (!row_ok) return;
+  float f = 1.0f / lrun;
+  if (a.gate) {
+    const bf16_t* gate = static_cast<const bf16_t*>(a.gate);
+    f *= 1.0f / (1.0f + expf(-bf2f(gate[row * a.gate_st + h])));
+  }
+  bf16_t* out = static_cast<bf16_t*>(a.out) + row * a.out_st + (long)h * a.out_sh;
+#pragma unroll
+  for (int ct = 0; ct < NCMAX; ++ct) {
+    if (ct < nc) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int col = ct * 16 + 4 * g + i;
+        if (col < a.R) out[col] = f2bf(acc[ct][i] * f);
+      }
+    }
+  }
+}
+
+// Rows per work item of the MFMA form: NW waves x 16; HB = min(H, 16) heads, QB = rows / HB
+// queries.  Returns QB for (H, prefill) so the host builds its work list with the same number.
+EIA_API int eia_latent_attn_mfma_qb(int H, int decode) {
+  const int HB = H < 16 ? H : 16;
+  return decode ? 1 : (64 / HB);
+}
+
+EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const void* qr,
+                                 long qr_st, long qr_sh, const float* inv_freq, int rot_dims,
+                                 const void* cache, long cache_row, const int* block_table,
+                                 int bt_stride, const int* seq_lens, const int* cu_q,
+                                 const int* work, int n_items, const int* positions,
+                                 const void* gate, long gate_st, void* out, long out_st,
+                                 long out_sh, float scale, int H, int R, int rd, int bs, int QB,
+                                 hipStream_t st) {
+  if (H < 1 || R < 1 || rd < 0 || bs < 1 || QB < 1 || rot_dims > rd || (rot_dims & 1) ||
+      cache_row < R + rd || (cu_q && !work))
+    return EIA_BAD_SHAPE;
+  const int Dk = R + rd;
+  // 16-byte chunks must not straddle the latent / rotary boundary or the row end
+  if ((R & 7) || (Dk & 7) || (cache_row & 7) || Dk > 640 || R > 512) return EIA_UNSUPPORTED;
+  if (n_items <= 0) return EIA_OK;
+  const int HB = H < 16 ? H : 16;
+  const bool decode = cu_q == nullptr;
+  if (QB != eia_latent_attn_mfma_qb(H, decode ? 1 : 0)) return EIA_BAD_SHAPE;
+  const int nk = (Dk + 31) / 32, Dkp = nk * 32, nc = (R + 15) / 16;
+  const int ldk = ((Dkp / 8) & 1) ? Dkp : Dkp + 8;       // odd number of 16-byte units per row
+  const size_t lds = ((size_t)32 * ldk + (size_t)nc * 16 * 40) * 2;
+  LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
+                   block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
+                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk};
+  dim3 grid(n_items, (H + HB - 1) / HB);
+#define LAT_MFMA(NK, NC, NW)                                                                \
+  do {                                                                                      \
+    if (lds > 48 * 1024)                                                                    \
+      (void)hipFuncSetAttribute(                                                            \
+          reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NK, NC, NW>),              \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                            \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<NK, NC, NW>), grid, dim3(NW * 64), lds, st, a); \
+  } while (0)
+  if (decode) {
+    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, 1);
+    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, 1);
+    else LAT_MFMA(20, 32, 1);
+  } else {
+    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, 4);
+    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, 4);
+    else LAT_MFMA(20, 32, 4);
+  }
+#undef LAT_MFMA
+  EIA_LAUNCH_CHECK();
+}

@@ -660,6 +660,9 @@ class ModelRunner:
             prefill_cu_q=d[o["cu"]:o["cu"] + npf + 1] if npf else None,
             prefill_work=d[o["work"]:o["work"] + 2 * nw] if npf else None,
             prefill_n_work=nw)
+        if npf:
+            md.prefill_qblock = self._query_block()
+            md.prefill_q_lens = np.diff(self.e_buf.numpy()[o["cu"]:o["cu"] + npf + 1]).tolist()
         if "sslot" in o:
             ns = nd + npf
             md.num_seqs = ns

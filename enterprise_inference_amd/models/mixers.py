@@ -75,7 +75,9 @@ class LatentAttentionMixer(nn.Module):
         self.uv = _plain((heads * vdim, kv_rank), dtype, device)
         self.o = _plain((width, heads * vdim), dtype, device)
         self.inv_freq = lat_ops.inv_frequencies(rot_dims, rot_base, device)
-        self.qblock = lat_ops.query_block(heads, kv_rank)
+        self.qblock = lat_ops.query_block(heads, kv_rank, rot_dim,
+                                          dtype if torch.device(device).type == "cuda"
+                                          else torch.float32)
 
     def _load_down(self, param, loaded, shard_id=None):
         off = {"dq": 0, "dkv": self.q_rank, "g": self.q_rank + self.kv_rows}[shard_id]
@@ -95,7 +97,7 @@ class LatentAttentionMixer(nn.Module):
         q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk.view(H, D, R)).transpose(0, 1)
         gate = fused[:, self.q_rank + self.kv_rows:]
         lat = lat_ops.latent_attention(q_abs, q[:, :, D:], self.inv_freq, self.rot_dims,
-                                       cache.rows, md, gate, self.scale, self.qblock)
+                                       cache.rows, md, gate, self.scale)
         # value up-projection of the attended latent, heads concatenated
         o = torch.bmm(lat.transpose(0, 1), self.uv.view(H, self.vdim, R).transpose(1, 2))
         return gemm.linear(o.transpose(0, 1).reshape(T, H * self.vdim), self.o)

@@ -140,8 +140,10 @@ class SekolornForCausalLM(nn.Module):
         return out
 
     def prefill_query_block(self, block_size: int) -> int:
-        qb = {L.mix.qblock for L in self.layers if L.kind == "latent_attention"}
-        return min(qb) if qb else 16
+        """The step's work list is built for the first latent layer's query block; layers with
+        another one get theirs from AttentionMetadata.prefill_work_for."""
+        qb = [L.mix.qblock for L in self.layers if L.kind == "latent_attention"]
+        return qb[0] if qb else 16
 
     # ------------------------------------------------------------------ forward
     def forward(self, input_ids: torch.Tensor, md: AttentionMetadata, caches: list,

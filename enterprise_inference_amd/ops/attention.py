@@ -153,6 +153,8 @@ class AttentionMetadata:
     prefill_cu_q: Optional[torch.Tensor] = None          # [Sp+1] int32
     prefill_work: Optional[torch.Tensor] = None          # [n_work*2] int32
     prefill_n_work: int = 0
+    prefill_qblock: int = 0                              # queries per work item (0: not stated)
+    prefill_q_lens: Optional[List[int]] = None           # host copy of the chunk lengths
     causal: bool = True
     # multimodal: batch rows whose token embedding is replaced (image placeholders)
     mm_rows: Optional[torch.Tensor] = None               # [n] int64
@@ -162,6 +164,25 @@ class AttentionMetadata:
     num_seqs: int = 0
     seq_slots: Optional[torch.Tensor] = None             # [num_seqs] int32 (< 0: padding row)
     seq_cu: Optional[torch.Tensor] = None                # [num_seqs + 1] int32
+    # work lists for kernels whose query block differs from prefill_qblock: qblock -> (list, n)
+    work_cache: dict = dataclasses.field(default_factory=dict)
+
+    def prefill_work_for(self, qblock: int, build):
+        """(work tensor, items) for a kernel that takes ``qblock`` queries per item: the step's
+        own list when it was built with that size, else one built (once per step and size) from
+        the chunk lengths with ``build(q_lens, qblock)``."""
+        if qblock == self.prefill_qblock and self.prefill_work is not None:
+            return self.prefill_work, self.prefill_n_work
+        hit = self.work_cache.get(qblock)
+        if hit is None:
+            lens = self.prefill_q_lens
+            if lens is None:
+                cu = self.prefill_cu_q.tolist()
+                lens = [cu[i + 1] - cu[i] for i in range(len(cu) - 1)]
+            w = build(lens, qblock)
+            hit = (torch.tensor(w, dtype=torch.int32, device=self.prefill_cu_q.device), len(w) // 2)
+            self.work_cache[qblock] = hit
+        return hit
 
     @property
     def num_tokens(self) -> int:

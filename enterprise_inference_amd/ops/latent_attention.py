@@ -12,6 +12,7 @@ cache after ``latent_prep`` wrote this step's rows, so chunked prompts need no s
 
 from __future__ import annotations
 
+import os
 from typing import List, Optional
 
 import torch
@@ -28,11 +29,25 @@ def inv_frequencies(dims: int, base: float, device) -> torch.Tensor:
         torch.float32).to(device)
 
 
-def query_block(num_heads: int, kv_rank: int) -> int:
-    """Queries per prefill work item: as many as the kernel's per-thread accumulators allow for
-    a 16-head slice (more queries per item = fewer passes over the cached keys)."""
+def mfma_ok(kv_rank: int, rot_dim: int, dtype: torch.dtype) -> bool:
+    """The MFMA kernel takes bf16 rows whose latent and total widths are multiples of 8 (its
+    16-byte chunks) up to 512 / 640; everything else runs the scalar-FMA kernel (fp32 too)."""
+    return (dtype == torch.bfloat16 and kv_rank % 8 == 0 and (kv_rank + rot_dim) % 8 == 0
+            and kv_rank <= 512 and kv_rank + rot_dim <= 640 and _MFMA_ENV)
+
+
+_MFMA_ENV = os.environ.get("EIA_LATENT_MFMA", "1") != "0"
+
+
+def query_block(num_heads: int, kv_rank: int, rot_dim: int = 0,
+                dtype: torch.dtype = torch.float32) -> int:
+    """Queries per prefill work item.  MFMA form: 64 (query, head) rows per workgroup in slices
+    of min(heads, 16) heads.  Scalar form: as many queries as the per-thread accumulators and
+    48 KiB of LDS for the staged queries allow for a 16-head slice."""
     hb = min(num_heads, 16)
-    return max(1, min(16, ACC_ROWS // (hb * kv_rank)))
+    if mfma_ok(kv_rank, rot_dim, dtype):
+        return 64 // hb
+    return max(1, min(16, ACC_ROWS // (hb * kv_rank), 12288 // (hb * (kv_rank + rot_dim))))
 
 
 def build_work(q_lens: List[int], qblock: int) -> List[int]:
@@ -129,12 +144,12 @@ def _ref_rows(q_abs, q_rot, inv_freq, rot_dims, cache, block_table, positions, g
 
 def latent_attention(q_abs: torch.Tensor, q_rot: torch.Tensor, inv_freq: torch.Tensor,
                      rot_dims: int, cache: torch.Tensor, md, gate: Optional[torch.Tensor],
-                     scale: float, qblock: int) -> torch.Tensor:
+                     scale: float) -> torch.Tensor:
     """q_abs [T, H, R] and q_rot [T, H, rd] (any strides with a contiguous last dim; q_rot not
     yet rotated), gate [T, H] pre-sigmoid or None -> latent output [T, H, R] (contiguous):
     softmax((q_abs . c + rot(q_rot) . k_rot) * scale) weighted sum of c, times sigmoid(gate).
-    ``md`` is the step's AttentionMetadata (decode rows first, then prefill chunks whose work
-    list was built with ``build_work(q_lens, qblock)``)."""
+    ``md`` is the step's AttentionMetadata (decode rows first, then prefill chunks; the work
+    list comes from ``md.prefill_work_for(query_block(...), build_work)``)."""
     T, H, R = q_abs.shape
     rd = q_rot.shape[-1]
     nd = md.num_decode
@@ -161,10 +176,20 @@ def latent_attention(q_abs: torch.Tensor, q_rot: torch.Tensor, inv_freq: torch.T
     require(md.positions.dtype == torch.int32, "positions int32")
     bs = cache.shape[1]
 
+    mfma = mfma_ok(R, rd, q_abs.dtype)
+
     def launch(lo, n_items, bt, lens, cu, work, qb):
         qa, qr, o = q_abs[lo:], q_rot[lo:], out[lo:]
         g = None if gate is None else gate[lo:]
         require(bt.dtype == torch.int32 and bt.stride(1) == 1, "block tables int32")
+        if mfma:
+            check(lib().eia_latent_attn_mfma(
+                ptr(qa), qa.stride(0), qa.stride(1), ptr(qr), qr.stride(0), qr.stride(1),
+                ptr(inv_freq), rot_dims, ptr(cache), cache.shape[-1], ptr(bt), bt.stride(0),
+                ptr(lens), ptr(cu), ptr(work), n_items, ptr(md.positions[lo:]), ptr(g),
+                g.stride(0) if g is not None else 0, ptr(o), o.stride(0), o.stride(1),
+                float(scale), H, R, rd, bs, qb, stream(q_abs)), "latent_attn_mfma")
+            return
         check(lib().eia_latent_attn(
             ptr(qa), qa.stride(0), qa.stride(1), ptr(qr), qr.stride(0), qr.stride(1),
             ptr(inv_freq), rot_dims, ptr(cache), cache.shape[-1], ptr(bt), bt.stride(0), ptr(lens),
@@ -175,6 +200,7 @@ def latent_attention(q_abs: torch.Tensor, q_rot: torch.Tensor, inv_freq: torch.T
     if nd:
         launch(0, nd, md.decode_block_tables, md.decode_seq_lens, None, None, 1)
     if md.num_prefill_tokens:
-        launch(nd, md.prefill_n_work, md.prefill_block_tables, None, md.prefill_cu_q,
-               md.prefill_work, qblock)
+        qb = query_block(H, R, rd, q_abs.dtype)
+        work, n_work = md.prefill_work_for(qb, build_work)
+        launch(nd, n_work, md.prefill_block_tables, None, md.prefill_cu_q, work, qb)
     return out

@@ -16,6 +16,12 @@ def tol(dtype):
     return 2e-4 if dtype == torch.float32 else 0.12
 
 
+def ktol(dtype):
+    """Kernel-level checks: inputs are already rounded to the dtype, so only the kernel's own
+    roundings (bf16 outputs, bf16 query / weight operands) remain."""
+    return 2e-4 if dtype == torch.float32 else 1.5e-2
+
+
 def _tokens(n, vocab, seed):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
@@ -52,7 +58,7 @@ def case_post_norm(device, dtype):
         assert torch.allclose(xb.float().cpu(), xd.cpu().to(dtype).float())
         out = norm.layer_norm_f32(xd, w.to(dtype).to(device), 1e-5)
         ref = O.layer_norm_nobias(xd.cpu().double(), w.to(dtype).double(), 1e-5)
-        assert torch.allclose(out.float().cpu().double(), ref, atol=tol(dtype), rtol=tol(dtype))
+        assert torch.allclose(out.float().cpu().double(), ref, atol=ktol(dtype), rtol=ktol(dtype))
 
 
 def case_route(device, dtype):
@@ -106,7 +112,7 @@ def case_ungated_moe(device, dtype):
             if e < E:
                 Wt = {"up": up[e].double(), "down": down[e].double()}
                 want += float(tw[t, s]) * O.expert(x[t].double(), Wt, "")
-        assert torch.allclose(out[t].double(), want, atol=tol(dtype) * 10, rtol=tol(dtype) * 10)
+        assert torch.allclose(out[t].double(), want, atol=ktol(dtype) * 4, rtol=ktol(dtype) * 4)
 
 
 def _paged(rows_c, rows_kr, block_size, nblocks, order, dtype, device):
@@ -119,14 +125,14 @@ def _paged(rows_c, rows_kr, block_size, nblocks, order, dtype, device):
     return cache.to(device)
 
 
-def case_latent_attention_needle(device, dtype):
+def case_latent_attention_needle(device, dtype, H=3, R=20, rd=6):
     """One far key is made to dominate one query's scores (its latent is aligned with the
     absorbed query and scaled up), at page borders and at the first positions: a mask or a
     block-table slip moves the output by O(1).  Decode rows and a prefill chunk in one step."""
     from enterprise_inference_amd.ops import latent_attention as la
     from enterprise_inference_amd.ops.attention import AttentionMetadata
     g = torch.Generator().manual_seed(4)
-    H, R, rd, bs, n = 3, 20, 6, 16, 83
+    bs, n = 16, 83
     rot_dims, base, scale = 4, 300.0, 0.4
     inv = la.inv_frequencies(rot_dims, base, device)
     c = torch.randn(n, R, generator=g).to(dtype).float()
@@ -162,12 +168,16 @@ def case_latent_attention_needle(device, dtype):
         prefill_block_tables=bt[None].to(device),
         prefill_seq_lens=torch.tensor([83], dtype=torch.int32, device=device),
         prefill_cu_q=torch.tensor([0, len(chunk)], dtype=torch.int32, device=device))
-    for qb in (1, 4, 16):
-        work = la.build_work([len(chunk)], qb)
-        md.prefill_work = torch.tensor(work, dtype=torch.int32, device=device)
-        md.prefill_n_work = len(work) // 2
+    for qb in (0, la.query_block(H, R, rd, dtype if device == "cuda" else torch.float32)):
+        # qb 0: the step states no work list (the op builds its own); else the step's list fits
+        md.work_cache.clear()
+        md.prefill_qblock = qb
+        if qb:
+            work = la.build_work([len(chunk)], qb)
+            md.prefill_work = torch.tensor(work, dtype=torch.int32, device=device)
+            md.prefill_n_work = len(work) // 2
         out = la.latent_attention(qa.to(device), qr.to(device), inv, rot_dims, cache, md,
-                                  gate.to(device), scale, qb).float().cpu()
+                                  gate.to(device), scale).float().cpu()
         for i, p in enumerate(rows):
             for h in range(H):
                 q_rot = O.rotate_interleaved(qr[i, h].double(), p, rot_dims, base)
@@ -175,8 +185,8 @@ def case_latent_attention_needle(device, dtype):
                                   * scale for j in range(p + 1)])
                 a = torch.softmax(s, 0)
                 want = (a[:, None] * c[:p + 1].double()).sum(0) * torch.sigmoid(gate[i, h].double())
-                assert torch.allclose(out[i, h].double(), want, atol=tol(dtype) * 5,
-                                      rtol=tol(dtype) * 5), (qb, i, p, h, needles[i])
+                assert torch.allclose(out[i, h].double(), want, atol=ktol(dtype) * 3,
+                                      rtol=ktol(dtype) * 3), (qb, i, p, h, needles[i])
 
 
 def case_latent_prep(device, dtype):
@@ -195,14 +205,14 @@ def case_latent_prep(device, dtype):
     f = fused.double()
     for t in range(T):
         want_q = O.rms_unit(f[t, :Q], 1e-5) * wq.double()
-        assert torch.allclose(cq[t].float().cpu().double(), want_q, atol=tol(dtype), rtol=tol(dtype))
+        assert torch.allclose(cq[t].float().cpu().double(), want_q, atol=ktol(dtype), rtol=ktol(dtype))
         if slots[t] < 0:
             continue
         want_c = O.rms_unit(f[t, Q:Q + R], 1e-5) * wc.double()
         want_k = O.rotate_interleaved(f[t, Q + R:Q + R + rd], int(pos[t]), rot_dims, base)
         got = flat[int(slots[t])].double()
-        assert torch.allclose(got[:R], want_c, atol=tol(dtype), rtol=tol(dtype))
-        assert torch.allclose(got[R:], want_k, atol=tol(dtype), rtol=tol(dtype))
+        assert torch.allclose(got[:R], want_c, atol=ktol(dtype), rtol=ktol(dtype))
+        assert torch.allclose(got[R:], want_k, atol=ktol(dtype), rtol=ktol(dtype))
     assert float(flat[5].abs().sum()) == 0.0          # the skipped row wrote nothing
 
 
@@ -246,8 +256,8 @@ def case_wkv(device, dtype):
                          S, prev, x, slots, cu, 2, pos, None, 1e-5, H).float().cpu().double()
         want = torch.cat([ya2, yb])
         scale = float(want.abs().max())
-        assert float((y - want).abs().max()) <= tol(dtype) * 20 * scale, (H, D)
-        t2 = tol(dtype) * 50
+        assert float((y - want).abs().max()) <= ktol(dtype) * 4 * scale, (H, D)
+        t2 = ktol(dtype) * 4
         assert torch.allclose(S[2].cpu().double(), st2["S"], atol=t2 * float(st2["S"].abs().max()))
         assert torch.allclose(S[0].cpu().double(), stb["S"], atol=t2 * float(stb["S"].abs().max()))
         assert torch.allclose(prev[2].cpu(), xa[8]) and torch.allclose(prev[0].cpu(), xb_[3])

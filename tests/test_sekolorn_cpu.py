@@ -19,6 +19,10 @@ def test_mechanism(case):
     case(DEV, DT)
 
 
+def test_latent_attention_more_heads():
+    K.case_latent_attention_needle(DEV, DT, 5, 24, 8)
+
+
 def test_schedules_config_a():
     K.case_schedules(DEV, DT, C.config_a)
 
