@@ -64,7 +64,16 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--mode", default="endpoint", choices=["endpoint", "engine"])
+    ap.add_argument("--mode", default="endpoint", choices=["endpoint", "engine", "design"],
+                    help="design: prefill / decode throughput of the Sekolorn design beside a "
+                         "Mixtral-style decoder at equal layer sizes (benchmarks/design_bench.py)")
+    ap.add_argument("--design-sizes", default="s,m", help="comma list of s, m, l")
+    ap.add_argument("--design-models", default="sekolorn,mixtral",
+                    help="which of the two engines to run (profiling one of them alone)")
+    ap.add_argument("--design-prompt-len", type=int, default=2048)
+    ap.add_argument("--design-prompts", type=int, default=4)
+    ap.add_argument("--design-users", type=int, default=32)
+    ap.add_argument("--design-gen", type=int, default=32)
     ap.add_argument("--model", default="meta-llama/Llama-3.1-8B-Instruct")
     ap.add_argument("--tp", type=int, default=1)
     ap.add_argument("--co-deploy", action="store_true",
@@ -891,6 +900,9 @@ def main() -> int:
     args = parse()
     if args.mode == "engine":
         return run_engine(args)
+    if args.mode == "design":
+        from benchmarks import design_bench
+        return design_bench.run(args)
     return run_endpoint(args)
 
 

@@ -1,0 +1,127 @@
+"""Prefill and decode throughput of one decoder design beside another at equal layer sizes
+(random weights, one GPU), through the offline engine: ``python bench.py --mode design``.
+
+For each size the two engines are built one after the other on the same device:
+* Sekolorn -- latent attention / wkv / latent attention reading the first layer's cache, each
+  with a group-routed ungated MoE and a shared expert;
+* the closest existing family, a Mixtral-style decoder (grouped-query attention + SwiGLU MoE)
+  with the same width, layer count, head count, head size, expert count, top-k and expert ff.
+Prefill: ``--design-prompts`` prompts of ``--design-prompt-len`` tokens, one sampled token each.
+Decode: ``--design-users`` sequences of 128 prompt tokens generating ``--design-gen`` tokens; the
+decode rate is the extra tokens over the extra time against the same run with one token.
+Prints one JSON line per (size, model) and a closing summary line.
+"""
+
+from __future__ import annotations
+
+import gc
+import json
+import time
+
+SIZES = {
+    # name: width, layers (multiple of 3), heads, head dim, rot dim, kv_rank, q_rank, wkv heads,
+    #       experts, top, groups, keep, ff, vocab
+    "s": dict(width=1024, layers=3, heads=8, dim=64, rot=32, kv_rank=128, q_rank=256,
+              wkv_heads=16, experts=8, top=2, groups=4, keep=2, ff=512, vocab=32000),
+    "m": dict(width=2048, layers=6, heads=16, dim=64, rot=32, kv_rank=256, q_rank=512,
+              wkv_heads=32, experts=16, top=2, groups=4, keep=2, ff=1024, vocab=32000),
+    "l": dict(width=4096, layers=6, heads=32, dim=128, rot=64, kv_rank=512, q_rank=1536,
+              wkv_heads=64, experts=16, top=4, groups=4, keep=2, ff=1536, vocab=32000),
+}
+
+
+def sekolorn_config(z: dict) -> dict:
+    def lat(kv_from=None):
+        m = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot"], "vdim": z["dim"],
+             "kv_rank": z["kv_rank"], "q_rank": z["q_rank"],
+             "scale": (z["dim"] + z["rot"]) ** -0.5, "rot": {"dims": z["rot"], "base": 10000.0}}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return m
+
+    def mlp():
+        return {"kind": "moe", "expert": {"ff": z["ff"]}, "shared": {"ff": z["ff"]},
+                "router": {"experts": z["experts"], "top": z["top"], "scale": 1.0,
+                           "groups": {"count": z["groups"], "keep": z["keep"]}}}
+
+    layers = []
+    for i in range(0, z["layers"], 3):
+        layers += [{"type": "latent_attention", "mixer": lat(), "mlp": mlp()},
+                   {"type": "wkv", "mixer": {"heads": z["wkv_heads"], "dim": 64, "decay_rank": 64},
+                    "mlp": mlp()},
+                   {"type": "latent_attention", "mixer": lat(kv_from=i), "mlp": mlp()}]
+    return {"architecture": "Sekolorn", "vocab": z["vocab"], "width": z["width"],
+            "norm": {"eps": 1e-6}, "layers": layers}
+
+
+def mixtral_config(z: dict) -> dict:
+    return {"architectures": ["MixtralForCausalLM"], "hidden_size": z["width"],
+            "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+            "num_key_value_heads": max(1, z["heads"] // 4), "head_dim": 128,
+            "vocab_size": z["vocab"], "intermediate_size": z["ff"],
+            "num_local_experts": z["experts"], "num_experts_per_tok": z["top"],
+            "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "rope_theta": 1e6}
+
+
+def _measure(cfg_dict: dict, a) -> dict:
+    import torch
+
+    from enterprise_inference_amd.config import (CacheConfig, EngineConfig, ModelConfig,
+                                                 SchedulerConfig)
+    from enterprise_inference_amd.engine.llm_engine import LLMEngine
+    from enterprise_inference_amd.engine.sampling_params import SamplingParams
+
+    P, NP, B, G = a.design_prompt_len, a.design_prompts, a.design_users, a.design_gen
+    ec = EngineConfig(model=ModelConfig.from_hf_dict(cfg_dict), device="cuda", load_format="dummy",
+                      cache=CacheConfig(block_size=128, num_gpu_blocks=max(
+                          NP * (P // 128 + 2), B * 4) + 8, swap_space_gb=0.0),
+                      scheduler=SchedulerConfig(max_num_seqs=max(B, NP),
+                                                max_num_batched_tokens=max(P, 2048),
+                                                max_model_len=P + 256),
+                      seed=a.seed)
+    eng = LLMEngine(ec)
+    V = cfg_dict.get("vocab", cfg_dict.get("vocab_size"))
+    g = torch.Generator().manual_seed(a.seed)
+
+    def prompts(n, length):
+        return torch.randint(1, V, (n, length), generator=g).tolist()
+
+    def run(pr, max_tokens):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        eng.generate(prompt_token_ids=pr, params=SamplingParams(max_tokens=max_tokens,
+                                                                temperature=0.0, ignore_eos=True))
+        torch.cuda.synchronize()
+        return time.time() - t0
+
+    run(prompts(2, P), 2)                                     # warm-up (library heuristics)
+    tp = min(run(prompts(NP, P), 1) for _ in range(a.steps))
+    dp = prompts(B, 128)
+    run(dp, 4)
+    t1 = min(run(dp, 1) for _ in range(a.steps))
+    t2 = min(run(dp, 1 + G) for _ in range(a.steps))
+    out = {"prefill_tok_s": NP * P / tp, "decode_tok_s": B * G / max(1e-9, t2 - t1),
+           "decode_ms_per_step": 1e3 * (t2 - t1) / G,
+           "graphs": bool(eng.executor.runner.graphs)}
+    eng.shutdown()
+    del eng
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def run(a) -> int:
+    rows = []
+    for name in a.design_sizes.split(","):
+        z = SIZES[name]
+        for label, cfg in (("Sekolorn", sekolorn_config(z)), ("Mixtral-style", mixtral_config(z))):
+            if label.split("-")[0].lower() not in a.design_models.lower():
+                continue
+            r = _measure(cfg, a)
+            r.update(size=name, model=label, width=z["width"], layers=z["layers"],
+                     prompt_len=a.design_prompt_len, users=a.design_users)
+            rows.append(r)
+            print(json.dumps(r), flush=True)
+    print(json.dumps({"metric": "design_comparison", "rows": rows, "dtype": "bf16",
+                      "data": "synthetic", "n_gpus": 1}), flush=True)
+    return 0

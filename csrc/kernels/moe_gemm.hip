@@ -33,7 +33,7 @@ template <bool SWIGLU>
 __global__ void __launch_bounds__(256, 2)
 moe_grouped_mfma_kernel(const bf16_t* __restrict__ X, long ldx, const int* __restrict__ row_idx,
                         const bf16_t* __restrict__ W, long w_estride, const int* __restrict__ offs,
-                        int E, int I, int K, bf16_t* __restrict__ out, long ldo) {
+                        int E, int I, int K, bf16_t* __restrict__ out, long ldo, int relu2) {
   extern __shared__ __align__(16) bf16_t lds[];
   __shared__ int s_e, s_m0;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -169,7 +169,11 @@ moe_grouped_mfma_kernel(const bf16_t* __restrict__ X, long ldx, const int* __res
         for (int j = 0; j < 4; ++j) {
           bf16x4 v;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = f2bf(acc[nt][mt][4 * j + r]);
+          for (int r = 0; r < 4; ++r) {
+            float x = acc[nt][mt][4 * j + r];
+            if (relu2) { x = fmaxf(x, 0.f); x *= x; }     // ungated experts: squared ReLU
+            v[r] = f2bf(x);
+          }
           *reinterpret_cast<bf16x4*>(op + c0 + 8 * j + 4 * h) = v;
         }
       }
@@ -182,12 +186,15 @@ moe_grouped_mfma_kernel(const bf16_t* __restrict__ X, long ldx, const int* __res
 // Grouped expert GEMM over the device-side expert slices of eia_moe_align.
 //   X [*, K] (ldx), rows gathered through row_idx (nullptr: identity); W [E][N][K] (expert
 //   stride N*K); out [rows_total][ldo] in sorted order.
-//   swiglu 1: N = 2I ([gate; up]), out has I columns; 0: out has N columns.
+//   swiglu 1: N = 2I ([gate; up]), out has I columns; 0: out has N columns; 2: N columns with
+//   a squared-ReLU epilogue (ungated experts' up projection).
 //   max_rows: host upper bound of offs[E] (T * top_k) -- sizes the grid.
 EIA_API int eia_moe_grouped_gemm(const void* X, long ldx, const int* row_idx, const void* W, int N,
                                  int K, int E, const int* offs, int max_rows, int swiglu, void* out,
                                  long ldo, hipStream_t st) {
   if (E < 1 || K % BK != 0 || (ldx % 8) || (ldo % 4)) return EIA_BAD_SHAPE;
+  const int relu2 = swiglu == 2;
+  if (relu2) swiglu = 0;
   if (swiglu ? (N % 2 != 0 || (N / 2) % 64 != 0) : (N % BN != 0)) return EIA_BAD_SHAPE;
   if (max_rows <= 0) return EIA_OK;
   static bool attr[2] = {false, false};
@@ -201,7 +208,7 @@ EIA_API int eia_moe_grouped_gemm(const void* X, long ldx, const int* row_idx, co
     }
     hipLaunchKernelGGL(moe_grouped_mfma_kernel<true>, grid, dim3(256), GG_LDS_BYTES, st,
                        (const bf16_t*)X, ldx, row_idx, (const bf16_t*)W, estr, offs, E, N / 2, K,
-                       (bf16_t*)out, ldo);
+                       (bf16_t*)out, ldo, 0);
   } else {
     if (!attr[0]) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(moe_grouped_mfma_kernel<false>),
@@ -210,7 +217,7 @@ EIA_API int eia_moe_grouped_gemm(const void* X, long ldx, const int* row_idx, co
     }
     hipLaunchKernelGGL(moe_grouped_mfma_kernel<false>, grid, dim3(256), GG_LDS_BYTES, st,
                        (const bf16_t*)X, ldx, row_idx, (const bf16_t*)W, estr, offs, E, 0, K,
-                       (bf16_t*)out, ldo);
+                       (bf16_t*)out, ldo, relu2);
   }
   EIA_LAUNCH_CHECK();
 }

@@ -228,8 +228,10 @@ class ModelRunner:
         #   ids[S] | pos[S] | slot[S] | len[S] | P (+3 pad) | src[S]
         # P: decode partitions of this step (read by K1 inside the graph); src: row of the
         # previous step's sampler output holding this row's input token (-1: host id)
-        self.hdr_len = 5 * S + 4
+        # recurrent-state models append  sslot[S]: the rows' state slots (-1: padding row)
+        self.hdr_len = 5 * S + 4 + (S if self.num_state_slots else 0)
         self.src_off = 4 * S + 4
+        self.sslot_off = 5 * S + 4
         # eager region: packed per step
         self.e_size = 3 * T + 2 * S * mb + 4 * S + 1 + 2 * self.max_work + S + 64 + \
             max(S, T) + 2 * S + 1
@@ -525,6 +527,10 @@ class ModelRunner:
         base = self.g_hdr.data_ptr()
         bm.native.build(seq_ids, starts, np.ones(n, dtype=np.int32), base + 4 * S, base + 8 * S,
                         self.g_bt.data_ptr(), self.maxb, base + 12 * S, S)
+        if self.num_state_slots:
+            so2 = self.sslot_off
+            hdr[so2:so2 + n] = [bm.state_slot(d.seq) for d in decodes]
+            hdr[so2 + n:so2 + Bp] = -1
         if Bp > n:
             hdr[n:Bp] = 0
             hdr[S + n:S + Bp] = 0
@@ -548,6 +554,9 @@ class ModelRunner:
             decode_seq_lens=d[3 * S:3 * S + Bp], decode_partitions=P, decode_part_o=self.part_o,
             decode_part_ml=self.part_ml, decode_part_cnt=self.part_cnt,
             decode_p_dyn=d[4 * S:4 * S + 1])
+        if self.num_state_slots:
+            md.num_seqs = Bp
+            md.seq_slots = d[self.sslot_off:self.sslot_off + Bp]
         return d[:Bp], md
 
     def _graph_forward(self, Bp: int, P: int) -> torch.Tensor:
@@ -1006,7 +1015,7 @@ class ModelRunner:
         hdr[2 * S:3 * S] = -1
         hdr[3 * S:4 * S] = 1
         hdr[4 * S] = 1
-        hdr[self.src_off:] = -1
+        hdr[self.src_off:] = -1            # also the state-slot region: every row a padding row
         self.d_g_hdr.copy_(hdr)
         self.d_g_bt.zero_()
         stream = torch.cuda.Stream()

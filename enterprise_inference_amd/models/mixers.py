@@ -123,7 +123,14 @@ class WKVMixer(nn.Module):
         self.u = _plain((heads, dim), dtype, device)
         self.norm = _plain((hd,), dtype, device)
         self.o = _plain((width, hd), dtype, device)
-        self._w2_f32: Optional[torch.Tensor] = None
+        # fp32 copy of W_w2 for the decay branch's last product; refreshed IN PLACE after a
+        # weight load (captured decode graphs hold its address)
+        self.w2_f32 = torch.zeros(hd, decay_rank, dtype=torch.float32, device=device)
+        self._w2_ready = False
+
+    def refresh(self) -> None:
+        self.w2_f32.copy_(self.w2)
+        self._w2_ready = True
 
     def _load_stream(self, param, loaded, shard_id=None):
         param.data[self.STREAMS.index(shard_id)].copy_(loaded)
@@ -138,9 +145,9 @@ class WKVMixer(nn.Module):
         # decay pre-activation: the low-rank branch ends in an fp32 product (what follows it --
         # bias, both exponentials -- is fp32 inside the scan)
         lo = torch.tanh(gemm.linear(mix[4], self.w1).float())
-        if self._w2_f32 is None or self._w2_f32.device != self.w2.device:
-            self._w2_f32 = self.w2.float()
-        dec = lo @ self._w2_f32.t()
+        if not self._w2_ready:
+            self.refresh()
+        dec = lo @ self.w2_f32.t()
         y = wkv_ops.wkv_scan(rkvg[0], rkvg[1], rkvg[2], rkvg[3], dec, self.w0, self.u.view(-1),
                              self.norm, state.S, state.prev, x, md.seq_slots, md.seq_cu,
                              md.num_seqs, md.positions,

@@ -80,7 +80,6 @@ class SekolornLayer(nn.Module):
 class SekolornForCausalLM(nn.Module):
     supports_pp = False
     supports_float32 = True        # every kernel of this model has an fp32 form
-    supports_graphs = False        # the expert GEMMs read their row offsets back per layer
     needs_state_slots = True
 
     def __init__(self, cfg: ModelConfig, dtype=torch.bfloat16, device=None):
@@ -104,6 +103,11 @@ class SekolornForCausalLM(nn.Module):
         self.head = _param((cfg.vocab_size, W), dtype, device)
         self.head.weight_loader = default_loader
         self.needs_state_slots = any(L.kind == "wkv" for L in self.layers)
+        # decode steps replay HIP graphs when every expert block has a device-side grouped form
+        # (bf16, width and expert ff multiples of 128); else they read row offsets back per layer
+        self.supports_graphs = dtype == torch.bfloat16 and all(
+            L.mlp is None or (W % 128 == 0 and L.mlp.w_up.shape[1] % 128 == 0)
+            for L in self.layers)
 
     # ------------------------------------------------------------------ cache geometry
     def kv_heads_per_rank(self) -> int:
@@ -239,4 +243,4 @@ class SekolornForCausalLM(nn.Module):
     def post_load(self) -> None:
         for L in self.layers:
             if L.kind == "wkv":
-                L.mix._w2_f32 = L.mix.w2.float()
+                L.mix.refresh()

@@ -327,6 +327,9 @@ def _fused_moe_per_expert(x, w13, w2, topk_w, topk_ids, e_lo, act):
     return out.to(x.dtype)
 
 
+UNGATED_GROUPED = os.environ.get("EIA_UNGATED_GROUPED", "1") != "0"
+
+
 def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: int,
                   keep_groups: int, route_scale: float,
                   row_len: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -388,6 +391,45 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
     dev = x.device
     st = stream(x)
     offs, row_idx, inv = _align(topk_ids, E, 0, E, n, dev, st)
+    capturing = torch.cuda.is_current_stream_capturing()
+    avg = n / E
+    bf = (x.dtype == torch.bfloat16 and w_up.is_contiguous() and w_down.is_contiguous()
+          and x.stride(1) == 1 and x.stride(0) % 8 == 0)
+    # device-side grouped forms (no host synchronisation, valid inside a HIP graph): the
+    # weight-streaming skinny kernel for decode-sized batches, the MFMA grouped kernel (squared
+    # ReLU in the up projection's epilogue) up to MFMA_MAX_ROWS rows per expert
+    if bf and H % 256 == 0 and I % 256 == 0 and avg <= 96 and UNGATED_GROUPED:
+        h1 = torch.empty(max(1, n), I, dtype=x.dtype, device=dev)
+        h2 = torch.empty(max(1, n), H, dtype=x.dtype, device=dev)
+        mt = max(1, min(8, -(-int(1.5 * n / E + 1) // 16)))
+        check(lib().eia_moe_gemm(ptr(x), x.stride(0), ptr(w_up), w_up.stride(1), None, ptr(h1),
+                                 h1.stride(0), I, H, E, ptr(offs), ptr(row_idx), mt, 0,
+                                 2 if I % 128 == 0 else 0, st), "moe_gemm_up")
+        h1 = activation.relu2(h1)
+        check(lib().eia_moe_gemm(ptr(h1), h1.stride(0), ptr(w_down), w_down.stride(1), None,
+                                 ptr(h2), h2.stride(0), H, I, E, ptr(offs), None, mt, 0,
+                                 2 if H % 128 == 0 else 0, st), "moe_gemm_down")
+        out = torch.empty(T, H, dtype=x.dtype, device=dev)
+        check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
+                                    ptr(out), out.stride(0), st), "moe_combine")
+        return out
+    if bf and H % 128 == 0 and I % 128 == 0 and (avg <= MFMA_MAX_ROWS or capturing) \
+            and UNGATED_GROUPED:
+        h1 = torch.empty(max(1, n), I, dtype=x.dtype, device=dev)
+        h2 = torch.empty(max(1, n), H, dtype=x.dtype, device=dev)
+        check(lib().eia_moe_grouped_gemm(ptr(x), x.stride(0), ptr(row_idx), ptr(w_up), I, H, E,
+                                         ptr(offs), n, 2, ptr(h1), h1.stride(0), st),
+              "moe_grouped_gemm_up_relu2")
+        check(lib().eia_moe_grouped_gemm(ptr(h1), h1.stride(0), None, ptr(w_down), H, I, E,
+                                         ptr(offs), n, 0, ptr(h2), h2.stride(0), st),
+              "moe_grouped_gemm_down")
+        out = torch.empty(T, H, dtype=x.dtype, device=dev)
+        check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
+                                    ptr(out), out.stride(0), st), "moe_combine")
+        return out
+    if capturing:
+        raise RuntimeError("ungated_moe: no host-sync-free form for this shape "
+                           "(bf16, H % 128 == 0 and I % 128 == 0 needed); run it eagerly")
     bounds = offs.tolist()                      # the one host synchronisation of this layer
     xs = x.index_select(0, row_idx[:bounds[E]].long())
     h1 = torch.empty(max(1, n), I, dtype=x.dtype, device=dev)

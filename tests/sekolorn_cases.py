@@ -92,17 +92,16 @@ def case_route_group_limit(device, dtype):
     assert abs(float(tw[0, 0]) - 1 / (1 + math.exp(-2.0))) < 1e-5
 
 
-def case_ungated_moe(device, dtype):
+def case_ungated_moe(device, dtype, E=5, I=12, H=24, T=11, k=2):
     from enterprise_inference_amd.ops import moe
     g = torch.Generator().manual_seed(3)
-    E, I, H, T, k = 5, 12, 24, 11, 2
     x = torch.randn(T, H, generator=g).to(dtype)
     up = (torch.randn(E, I, H, generator=g) / H ** 0.5).to(dtype)
     down = (torch.randn(E, H, I, generator=g) / I ** 0.5).to(dtype)
     ids = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
-    ids[3, 1] = E                                            # routes nowhere
+    ids[3, k - 1] = E                                        # routes nowhere
     tw = torch.rand(T, k, generator=g)
-    tw[3, 1] = 0.0
+    tw[3, k - 1] = 0.0
     out = moe.ungated_moe(x.to(device), up.to(device), down.to(device), tw.to(device),
                           ids.to(device)).float().cpu()
     for t in range(T):
@@ -357,7 +356,7 @@ def case_long_decode(device, dtype, cfg_fn=C.config_b):
         sess.close()
 
 
-def case_generate(device, dtype, cfg_fn=C.config_a):
+def case_generate(device, dtype, cfg_fn=C.config_a, expect_graphs=None):
     """Greedy generation through LLMEngine (its scheduler, batching and sampler): every emitted
     token is the oracle's argmax given the tokens before it, for unequal prompts in one batch."""
     import copy
@@ -377,6 +376,8 @@ def case_generate(device, dtype, cfg_fn=C.config_a):
     model = eng.executor.runner.model
     model.load_weights(W.items())
     model.post_load()
+    if expect_graphs is not None:
+        assert bool(eng.executor.runner.graphs) == expect_graphs
     prompts = [_tokens(n, cfg["vocab"], 30 + n) for n in (40, 7, 1, 19)]     # 4 prompts, 3 slots
     outs = eng.generate(prompt_token_ids=prompts,
                         params=SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True))

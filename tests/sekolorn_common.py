@@ -57,6 +57,22 @@ def config_b():
             ]}
 
 
+def config_c():
+    """Width and expert sizes in multiples of 128: bf16 engines run the experts' device-side
+    grouped forms and replay decode steps from HIP graphs."""
+    return {"architecture": "Sekolorn", "vocab": 160, "width": 128, "norm": {"eps": 1e-5},
+            "layers": [
+                {"type": "latent_attention",
+                 "mixer": latent(heads=4, dim=16, rot_dim=8, vdim=16, kv_rank=32, q_rank=32),
+                 "mlp": moe(experts=4, top=2, count=2, keep=1, ff=128, shared=128)},
+                {"type": "wkv", "mixer": {"heads": 2, "dim": 32, "decay_rank": 8},
+                 "mlp": moe(experts=4, top=2, count=2, keep=1, ff=128, shared=0)},
+                {"type": "latent_attention",
+                 "mixer": latent(heads=4, dim=16, rot_dim=8, vdim=16, kv_rank=32, q_rank=32,
+                                 kv_from=0), "mlp": None},
+            ]}
+
+
 def all_experts(cfg: dict) -> dict:
     """The same model with every expert of every group chosen.  With bf16 activations a
     router score that nearly ties another can pick a different expert than the float64 oracle

@@ -39,6 +39,10 @@ def test_generate_through_engine():
     K.case_generate(DEV, DT)
 
 
+def test_generate_config_c():
+    K.case_generate(DEV, DT, C.config_c)
+
+
 def test_state_slots_pool():
     from enterprise_inference_amd.engine.block_manager import StateSlots
     s = StateSlots(3)

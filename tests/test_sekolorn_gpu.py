@@ -35,6 +35,15 @@ def test_latent_attention_shapes(shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+@pytest.mark.parametrize("shape", [(4, 256, 256, 9, 2), (4, 128, 128, 40, 2), (3, 256, 256, 230, 2),
+                                   (2, 128, 256, 300, 1)], ids=lambda s: "x".join(map(str, s)))
+def test_ungated_moe_forms(shape, dtype):
+    """(E, I, H, T, k) that select, in bf16, the grouped weight-streaming form, the grouped MFMA
+    form (both without a host read-back) and the per-expert library form."""
+    K.case_ungated_moe("cuda", dtype, *shape)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_schedules_config_a(dtype):
     K.case_schedules("cuda", dtype, _cfg(C.config_a, dtype))
 
@@ -52,6 +61,14 @@ def test_long_decode(dtype):
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_generate_through_engine(dtype):
     K.case_generate("cuda", dtype, _cfg(C.config_a, dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_generate_graph_decode(dtype):
+    """A graph-eligible configuration: the bf16 engine captures decode graphs (state slots and
+    block tables are read from the graph's header on every replay); every decoded token of
+    every replay is checked against the oracle."""
+    K.case_generate("cuda", dtype, _cfg(C.config_c, dtype), expect_graphs=dtype == torch.bfloat16)
 
 
 def test_native_library_loaded():
