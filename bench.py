@@ -70,6 +70,9 @@ def parse():
     ap.add_argument("--design-sizes", default="s,m", help="comma list of s, m, l")
     ap.add_argument("--design-models", default="sekolorn,mixtral",
                     help="which of the two engines to run (profiling one of them alone)")
+    ap.add_argument("--design-kernels", action="store_true",
+                    help="design mode: time the design's attention / scan kernels beside the "
+                         "like kernels of the Llama path instead of whole engines")
     ap.add_argument("--design-prompt-len", type=int, default=2048)
     ap.add_argument("--design-prompts", type=int, default=4)
     ap.add_argument("--design-users", type=int, default=32)
@@ -902,7 +905,7 @@ def main() -> int:
         return run_engine(args)
     if args.mode == "design":
         from benchmarks import design_bench
-        return design_bench.run(args)
+        return design_bench.kernel_rates(args) if args.design_kernels else design_bench.run(args)
     return run_endpoint(args)
 
 

@@ -125,3 +125,114 @@ def run(a) -> int:
     print(json.dumps({"metric": "design_comparison", "rows": rows, "dtype": "bf16",
                       "data": "synthetic", "n_gpus": 1}), flush=True)
     return 0
+
+
+# ---------------------------------------------------------------------------------- kernel rates
+def _time(fn, iters: int = 5) -> float:
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    best = 1e9
+    for _ in range(iters):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) * 1e-3)
+    return best
+
+
+def kernel_rates(a) -> int:
+    """Achieved rates of the new design's kernels beside the like kernels of the Llama / Mixtral
+    path at equal head counts and lengths (``--design-kernels``): causal prefill attention
+    (useful TFLOP/s: 2 (Dqk + Dv) per query-key pair and head, the hi/lo second product of the
+    latent kernel not counted), decode attention (cache bytes read per second) and the wkv scan
+    (tokens/s and state bytes/s).  One JSON line per kernel."""
+    import torch
+
+    from enterprise_inference_amd.ops import attention as A
+    from enterprise_inference_amd.ops import latent_attention as LA
+    from enterprise_inference_amd.ops import wkv as WK
+
+    dev, bf = "cuda", torch.bfloat16
+    bs = 128
+    rows = []
+    for (H, R, rd, T) in ((8, 128, 32, 4096), (16, 512, 64, 4096)):
+        nb = T // bs
+        cache = torch.randn(nb, bs, R + rd, device=dev).to(bf)
+        qa = torch.randn(T, H, R, device=dev).to(bf) * 0.1
+        qr = torch.randn(T, H, rd, device=dev).to(bf) * 0.1
+        inv = LA.inv_frequencies(rd, 10000.0, dev)
+        bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+        pos = torch.arange(T, dtype=torch.int32, device=dev)
+        qb = LA.query_block(H, R, rd, bf)
+        work = LA.build_work([T], qb)
+        md = A.AttentionMetadata(
+            num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
+            prefill_block_tables=bt, prefill_seq_lens=torch.tensor([T], dtype=torch.int32, device=dev),
+            prefill_cu_q=torch.tensor([0, T], dtype=torch.int32, device=dev),
+            prefill_work=torch.tensor(work, dtype=torch.int32, device=dev),
+            prefill_n_work=len(work) // 2, prefill_qblock=qb)
+        t = _time(lambda: LA.latent_attention(qa, qr, inv, rd, cache, md, None, 0.1))
+        fl = 2.0 * (2 * R + rd) * H * T * (T + 1) / 2
+        rows.append({"kernel": "latent_attn_mfma prefill", "heads": H, "kv_rank": R, "rot": rd,
+                     "tokens": T, "ms": t * 1e3, "tflops": fl / t / 1e12})
+        # the like kernel: paged flash prefill, same heads, D = 128, GQA group 4
+        D, Hkv = 128, max(1, H // 4)
+        kc = torch.randn(nb, Hkv, bs, D, device=dev).to(bf)
+        vc = torch.randn(nb, Hkv, D, bs, device=dev).to(bf)
+        q = torch.randn(T, H, D, device=dev).to(bf) * 0.1
+        qb2 = A.prefill_query_block(H, Hkv, D, block_size=bs)
+        w2 = A.build_prefill_work([T], qb2)
+        t2 = _time(lambda: A.paged_prefill(q, kc, vc, bt, md.prefill_seq_lens, md.prefill_cu_q,
+                                           torch.tensor(w2, dtype=torch.int32, device=dev),
+                                           len(w2) // 2, 0.1))
+        rows.append({"kernel": "paged_prefill (flash)", "heads": H, "head_dim": D, "tokens": T,
+                     "ms": t2 * 1e3, "tflops": 2.0 * 2 * D * H * T * (T + 1) / 2 / t2 / 1e12})
+        # decode: B sequences of context L
+        B, L = 64, 4096
+        nbd = B * L // bs
+        cache_d = torch.randn(nbd, bs, R + rd, device=dev).to(bf)
+        btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
+        posd = torch.full((B,), L - 1, dtype=torch.int32, device=dev)
+        lens = torch.full((B,), L, dtype=torch.int32, device=dev)
+        mdd = A.AttentionMetadata(num_decode=B, num_prefill_tokens=0, slot_mapping=posd,
+                                  positions=posd, decode_block_tables=btd, decode_seq_lens=lens)
+        qad, qrd = qa[:B].contiguous(), qr[:B].contiguous()
+        t3 = _time(lambda: LA.latent_attention(qad, qrd, inv, rd, cache_d, mdd, None, 0.1))
+        rows.append({"kernel": "latent_attn_mfma decode", "heads": H, "kv_rank": R, "batch": B,
+                     "context": L, "ms": t3 * 1e3,
+                     "cache_GBps": B * L * (R + rd) * 2 / t3 / 1e9})
+        kcd = torch.randn(nbd, Hkv, bs, D, device=dev).to(bf)
+        vcd = torch.randn(nbd, Hkv, D, bs, device=dev).to(bf)
+        qd = q[:B].contiguous()
+        t4 = _time(lambda: A.paged_decode(qd, kcd, vcd, btd, lens, 0.1))
+        rows.append({"kernel": "paged_decode", "heads": H, "kv_heads": Hkv, "batch": B,
+                     "context": L, "ms": t4 * 1e3,
+                     "cache_GBps": B * L * Hkv * D * 2 * 2 / t4 / 1e9})
+    # wkv: one long prompt (sequential scan) and a decode batch (state traffic)
+    Hh, D, W = 32, 64, 2048
+    for (nseq, per) in ((1, 4096), (64, 1)):
+        T = nseq * per
+        HD = Hh * D
+        r, k, v, g = (torch.randn(T, HD, device=dev).to(bf) * 0.3 for _ in range(4))
+        dec = torch.randn(T, HD, device=dev) * 0.3
+        w0 = torch.full((HD,), -1.0, device=dev).to(bf)
+        u = (torch.randn(HD, device=dev) * 0.3).to(bf)
+        nw = torch.ones(HD, device=dev).to(bf)
+        S = torch.zeros(nseq, Hh, D, D, device=dev)
+        prev = torch.zeros(nseq, W, device=dev)
+        x = torch.randn(T, W, device=dev)
+        slots = torch.arange(nseq, dtype=torch.int32, device=dev)
+        cu = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
+        pos = (torch.arange(T, dtype=torch.int32, device=dev) % per) + (5 if per == 1 else 0)
+        t5 = _time(lambda: WK.wkv_scan(r, k, v, g, dec, w0, u, nw, S, prev, x, slots, cu, nseq,
+                                       pos, None, 1e-5, Hh))
+        rows.append({"kernel": "wkv_scan", "heads": Hh, "dim": D, "seqs": nseq, "tokens_per_seq": per,
+                     "ms": t5 * 1e3, "tokens_per_s": T / t5,
+                     "state_GBps": nseq * Hh * D * D * 4 * 2 / t5 / 1e9})
+    for r_ in rows:
+        print(json.dumps(r_), flush=True)
+    print(json.dumps({"metric": "design_kernel_rates", "rows": rows}), flush=True)
+    return 0

@@ -101,6 +101,9 @@ struct LatentAttnArgs {
   const void* gate; long gate_st;           // nullable: sigmoid(gate[t][h]) scales head h
   void* out; long out_st, out_sh;           // (t, h, r)
   float scale; int H, R, rd, bs, QB, HB, KC, ldk;
+  // MFMA decode only: the keys of a row split over grid.z partitions; each writes its
+  // unnormalised accumulators and (running max in log2 units, sum) for the merge kernel
+  int nparts; float* part_acc; float* part_ml;
 };
 
 template <typename T>
@@ -292,7 +295,7 @@ EIA_API int eia_latent_attn(const void* qa, long qa_st, long qa_sh, const void* 
   if (lds > 150 * 1024) return EIA_UNSUPPORTED;
   LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
                    block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
-                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, KC, ldk};
+                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, KC, ldk, 1, nullptr, nullptr};
   dim3 grid(n_items, (H + HB - 1) / HB);
   if (is_bf16) {
     if (lds > 48 * 1024)
@@ -318,7 +321,11 @@ EIA_API int eia_latent_attn(const void* qa, long qa_st, long qa_sh, const void* 
 // of the second product (no shuffle, no LDS round trip for P).  Softmax weights stay fp32: P
 // is fed as a bf16 high part plus a bf16 remainder (two MFMAs), and the normaliser sums the
 // fp32 weights.  The next unit's cache rows are prefetched into registers during the products.
-template <int NKMAX, int NCMAX, int NW>
+// SPLITV (decode, one query): all NW waves own the SAME 16 rows (the heads of one query) and
+// each takes every NW-th latent column tile of the second product; the first product is
+// repeated per wave (decode is bound by the cache stream, not by MFMA issue), which buys NW
+// times the loading threads (so the prefetch fits) and a quarter of the accumulators.
+template <int NKMAX, int NCMAX, int NW, bool SPLITV>
 __global__ void __launch_bounds__(NW * 64)
 latent_attn_mfma_kernel(LatentAttnArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -352,7 +359,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   const int* bt = a.block_table + (long)seq * a.bt_stride;
 
   // this lane's row (B operand column / accumulator column)
-  const int m = wave * 16 + c;
+  const int m = SPLITV ? c : wave * 16 + c;
   const int t = m / a.HB, h = h0 + (m - t * a.HB);
   const bool row_ok = t < ntok && h < a.H && m < a.QB * a.HB;
   const long row = row0 + (row_ok ? t : 0);
@@ -386,12 +393,21 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
       }
     }
   }
-  f32x4 acc[NCMAX];
+  constexpr int NACC = SPLITV ? (NCMAX + NW - 1) / NW : NCMAX;   // column tiles of this wave
+  const int ct0 = SPLITV ? wave : 0, ctstep = SPLITV ? NW : 1;   // tile i -> ct0 + i * ctstep
+  f32x4 acc[NACC];
 #pragma unroll
-  for (int i = 0; i < NCMAX; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < NACC; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
   float mrun = -INFINITY, lrun = 0.f;
   const float scale_log2 = a.scale * 1.4426950408889634f;
   const int kmax = a.positions[row0 + ntok - 1] + 1;
+  int k_begin = 0, k_end = kmax;
+  if (a.nparts > 1) {                                      // this partition's run of 32-key units
+    const int units = (kmax + 31) >> 5;
+    const int per = (units + a.nparts - 1) / a.nparts;
+    k_begin = min((int)blockIdx.z * per, units) << 5;
+    k_end = min(kmax, ((int)blockIdx.z + 1) * per << 5);
+  }
   const int cpr = Dkp >> 3;                                // 16-byte chunks per (padded) key row
   const int nchunk = 32 * cpr;
 
@@ -399,7 +415,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
     const int j = ch / cpr, d = (ch - j * cpr) << 3;
     const int kp = k0 + j;
-    if (kp < kmax && d < Dk) {                             // Dk % 8 == 0: whole chunk inside
+    if (kp < k_end && d < Dk) {                            // Dk % 8 == 0: whole chunk inside
       const long slot = (long)bt[kp / a.bs] * a.bs + (kp % a.bs);
       v = *reinterpret_cast<const bf16x8*>(cache + slot * a.cache_row + d);
     }
@@ -421,8 +437,8 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
       }
     }
   };
-  fetch(0);
-  for (int k0 = 0; k0 < kmax; k0 += 32) {
+  fetch(k_begin);
+  for (int k0 = k_begin; k0 < k_end; k0 += 32) {
     if constexpr (PREFETCH) {
 #pragma unroll
       for (int i = 0; i < PRE; ++i) {
@@ -443,7 +459,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
       for (int e = 0; e < 8; ++e) vt[(d + e) * LDV + j] = v[e];
     }
     __syncthreads();
-    if (k0 + 32 < kmax) fetch(k0 + 32);
+    if (k0 + 32 < k_end) fetch(k0 + 32);
     // S^T tiles: keys (rows) x this wave's 16 rows (columns)
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -486,18 +502,39 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     mrun = mnew;
     const bool rescale = !__all(alpha == 1.f);
 #pragma unroll
-    for (int ct = 0; ct < NCMAX; ++ct) {
+    for (int ai = 0; ai < NACC; ++ai) {
+      const int ct = ct0 + ai * ctstep;
       if (ct < nc) {
         const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vt + (ct * 16 + c) * LDV + 8 * g);
-        f32x4 o = acc[ct];
+        f32x4 o = acc[ai];
         if (rescale) o *= alpha;
         o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph, o, 0, 0, 0);
-        acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o, 0, 0, 0);
+        acc[ai] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl, o, 0, 0, 0);
       }
     }
     __syncthreads();
   }
   if (!row_ok) return;
+  if (a.nparts > 1) {
+    const long pr = ((long)row * a.H + h) * a.nparts + blockIdx.z;
+    float* pa = a.part_acc + pr * a.R;
+#pragma unroll
+    for (int ai = 0; ai < NACC; ++ai) {
+      const int ct = ct0 + ai * ctstep;
+      if (ct < nc) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int col = ct * 16 + 4 * g + i;
+          if (col < a.R) pa[col] = acc[ai][i];
+        }
+      }
+    }
+    if (g == 0 && (!SPLITV || wave == 0)) {
+      a.part_ml[2 * pr] = mrun;
+      a.part_ml[2 * pr + 1] = lrun;
+    }
+    return;
+  }
   float f = 1.0f / lrun;
   if (a.gate) {
     const bf16_t* gate = static_cast<const bf16_t*>(a.gate);
@@ -505,14 +542,43 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   }
   bf16_t* out = static_cast<bf16_t*>(a.out) + row * a.out_st + (long)h * a.out_sh;
 #pragma unroll
-  for (int ct = 0; ct < NCMAX; ++ct) {
+  for (int ai = 0; ai < NACC; ++ai) {
+    const int ct = ct0 + ai * ctstep;
     if (ct < nc) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int col = ct * 16 + 4 * g + i;
-        if (col < a.R) out[col] = f2bf(acc[ct][i] * f);
+        if (col < a.R) out[col] = f2bf(acc[ai][i] * f);
       }
     }
+  }
+}
+
+// Merge of the decode partitions: out = sum_p acc_p 2^(m_p - M) / sum_p l_p 2^(m_p - M), times
+// the head gate.  One workgroup per (row, head), threads over the latent columns.
+__global__ void __launch_bounds__(128)
+latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                    int nparts, const int* __restrict__ seq_lens, const bf16_t* __restrict__ gate,
+                    long gate_st, bf16_t* __restrict__ out, long out_st, long out_sh, int H, int R) {
+  const int row = blockIdx.x, h = blockIdx.y;
+  if (seq_lens && seq_lens[row] <= 0) return;
+  const long pr = ((long)row * H + h) * nparts;
+  float M = -INFINITY;
+  for (int p = 0; p < nparts; ++p) M = fmaxf(M, part_ml[2 * (pr + p)]);
+  float L = 0.f;
+  for (int p = 0; p < nparts; ++p) {
+    const float m = part_ml[2 * (pr + p)];
+    if (m != -INFINITY) L += part_ml[2 * (pr + p) + 1] * exp2f(m - M);
+  }
+  float f = L > 0.f ? 1.0f / L : 0.f;
+  if (gate) f *= 1.0f / (1.0f + expf(-bf2f(gate[row * gate_st + h])));
+  for (int c = threadIdx.x; c < R; c += blockDim.x) {
+    float v = 0.f;
+    for (int p = 0; p < nparts; ++p) {
+      const float m = part_ml[2 * (pr + p)];
+      if (m != -INFINITY) v += part_acc[(pr + p) * R + c] * exp2f(m - M);
+    }
+    out[row * out_st + h * out_sh + c] = f2bf(v * f);
   }
 }
 
@@ -530,7 +596,7 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
                                  const int* work, int n_items, const int* positions,
                                  const void* gate, long gate_st, void* out, long out_st,
                                  long out_sh, float scale, int H, int R, int rd, int bs, int QB,
-                                 hipStream_t st) {
+                                 int nparts, float* part_acc, float* part_ml, hipStream_t st) {
   if (H < 1 || R < 1 || rd < 0 || bs < 1 || QB < 1 || rot_dims > rd || (rot_dims & 1) ||
       cache_row < R + rd || (cu_q && !work))
     return EIA_BAD_SHAPE;
@@ -541,30 +607,37 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
   const int HB = H < 16 ? H : 16;
   const bool decode = cu_q == nullptr;
   if (QB != eia_latent_attn_mfma_qb(H, decode ? 1 : 0)) return EIA_BAD_SHAPE;
+  if (nparts < 1 || nparts > 64 || (nparts > 1 && (!decode || !part_acc || !part_ml)))
+    return EIA_BAD_SHAPE;
   const int nk = (Dk + 31) / 32, Dkp = nk * 32, nc = (R + 15) / 16;
   const int ldk = ((Dkp / 8) & 1) ? Dkp : Dkp + 8;       // odd number of 16-byte units per row
   const size_t lds = ((size_t)32 * ldk + (size_t)nc * 16 * 40) * 2;
   LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
                    block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
-                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk};
-  dim3 grid(n_items, (H + HB - 1) / HB);
-#define LAT_MFMA(NK, NC, NW)                                                                \
+                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk, nparts, part_acc,
+                   part_ml};
+  dim3 grid(n_items, (H + HB - 1) / HB, nparts);
+#define LAT_MFMA(NK, NC, SV)                                                                \
   do {                                                                                      \
     if (lds > 48 * 1024)                                                                    \
       (void)hipFuncSetAttribute(                                                            \
-          reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NK, NC, NW>),              \
+          reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NK, NC, 4, SV>),           \
           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                            \
-    hipLaunchKernelGGL((latent_attn_mfma_kernel<NK, NC, NW>), grid, dim3(NW * 64), lds, st, a); \
+    hipLaunchKernelGGL((latent_attn_mfma_kernel<NK, NC, 4, SV>), grid, dim3(256), lds, st, a); \
   } while (0)
   if (decode) {
-    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, 1);
-    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, 1);
-    else LAT_MFMA(20, 32, 1);
+    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, true);
+    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, true);
+    else LAT_MFMA(20, 32, true);
   } else {
-    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, 4);
-    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, 4);
-    else LAT_MFMA(20, 32, 4);
+    if (nk <= 6 && nc <= 8) LAT_MFMA(6, 8, false);
+    else if (nk <= 12 && nc <= 16) LAT_MFMA(12, 16, false);
+    else LAT_MFMA(20, 32, false);
   }
 #undef LAT_MFMA
+  if (nparts > 1)
+    hipLaunchKernelGGL(latent_merge_kernel, dim3(n_items, H), dim3(128), 0, st, part_acc, part_ml,
+                       nparts, seq_lens, static_cast<const bf16_t*>(gate), gate_st,
+                       static_cast<bf16_t*>(out), out_st, out_sh, H, R);
   EIA_LAUNCH_CHECK();
 }

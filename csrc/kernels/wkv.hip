@@ -75,64 +75,91 @@ struct WkvArgs {
 };
 
 // One workgroup per (sequence, head); thread j owns column j of S (dk values in registers,
-// DMAX >= D) and walks the sequence's tokens in order.
+// DMAX >= D) and walks the sequence's tokens in order.  Tokens are staged TC at a time: every
+// thread loads its channel of r, k, decay, v and the gate for TC tokens (coalesced over the
+// channels), r / k / w go to LDS, and the recurrence then runs TC steps on LDS broadcasts, so a
+// token costs one pass over dk instead of a global-memory round trip.
+#define WKV_TC (DMAX > 128 ? 8 : 16)
+
 template <typename T, int DMAX>
 __global__ void __launch_bounds__(DMAX < 64 ? 64 : DMAX)
 wkv_scan_kernel(WkvArgs a) {
-  __shared__ float sr[DMAX], sk[DMAX], sw[DMAX], su[DMAX], red[4];
+  // channels >= D hold zeros, so the dk loops below run branch-free over DMAX
+  __shared__ __align__(16) float sr[WKV_TC][DMAX], sk[WKV_TC][DMAX], sw[WKV_TC][DMAX], su[DMAX];
+  __shared__ float sv[WKV_TC][DMAX], sg[WKV_TC][DMAX];
+  __shared__ float red[4];
   const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x, D = a.D;
   const int slot = a.slots[s];
   if (slot < 0 || (a.seq_lens && a.seq_lens[s] <= 0)) return;
   const int lo = a.cu ? a.cu[s] : s, hi = a.cu ? a.cu[s + 1] : s + 1;
   if (hi <= lo) return;
   const bool fresh = a.positions[lo] == 0;
+  const bool live = j < D, mine = j < DMAX;
   float* Sg = a.S + ((long)slot * a.H + h) * D * D;
   float S[DMAX];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && i < D && j < D) ? Sg[(long)i * D + j] : 0.f;
+  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && i < D && live) ? Sg[(long)i * D + j] : 0.f;
   const long hc = (long)h * D;
-  if (j < D) su[j] = ld_f32<T>(static_cast<const T*>(a.u), hc + j);
-  const float w0 = j < D ? ld_f32<T>(static_cast<const T*>(a.w0), hc + j) : 0.f;
-  const float nw = j < D ? ld_f32<T>(static_cast<const T*>(a.norm_w), hc + j) : 0.f;
+  if (mine) su[j] = live ? ld_f32<T>(static_cast<const T*>(a.u), hc + j) : 0.f;
+  const float w0 = live ? ld_f32<T>(static_cast<const T*>(a.w0), hc + j) : 0.f;
+  const float nw = live ? ld_f32<T>(static_cast<const T*>(a.norm_w), hc + j) : 0.f;
   const T* R = static_cast<const T*>(a.r);
   const T* K = static_cast<const T*>(a.k);
   const T* V = static_cast<const T*>(a.v);
   const T* G = static_cast<const T*>(a.g);
   T* Y = static_cast<T*>(a.y);
-  for (int row = lo; row < hi; ++row) {
-    __syncthreads();
-    float vj = 0.f;
-    if (j < D) {
-      sr[j] = ld_f32<T>(R, row * a.ld + hc + j);
-      sk[j] = ld_f32<T>(K, row * a.ld + hc + j);
-      sw[j] = expf(-expf(a.dec[row * a.ld_dec + hc + j] + w0));
-      vj = ld_f32<T>(V, row * a.ld + hc + j);
-    }
-    __syncthreads();
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < DMAX; ++i) {
-      if (i < D) {
-        const float kv = sk[i] * vj;
-        o += sr[i] * (S[i] + su[i] * kv);
-        S[i] = sw[i] * S[i] + kv;
+  constexpr int NWV = (DMAX + 63) / 64;
+  const float inv_d = 1.0f / (float)D;
+  for (int base = lo; base < hi; base += WKV_TC) {
+    const int nt = min(WKV_TC, hi - base);
+    __syncthreads();                       // the previous chunk's LDS reads are done
+    if (mine) {
+#pragma unroll 4
+      for (int t = 0; t < nt; ++t) {
+        const long row = base + t;
+        float r = 0.f, k = 0.f, w = 0.f, v = 0.f, g = 0.f;
+        if (live) {
+          r = ld_f32<T>(R, row * a.ld + hc + j);
+          k = ld_f32<T>(K, row * a.ld + hc + j);
+          w = expf(-expf(a.dec[row * a.ld_dec + hc + j] + w0));
+          v = ld_f32<T>(V, row * a.ld + hc + j);
+          g = ld_f32<T>(G, row * a.ld + hc + j);
+        }
+        sr[t][j] = r;
+        sk[t][j] = k;
+        sw[t][j] = w;
+        sv[t][j] = v;
+        sg[t][j] = g;
       }
     }
-    // head RMS norm over the D outputs, then channel weight and gate
-    float ss = wave_sum(j < D ? o * o : 0.f);
-    if (DMAX > 64) {
-      if ((j & 63) == 0) red[j >> 6] = ss;
-      __syncthreads();
-      ss = 0.f;
-      for (int q = 0; q < (DMAX + 63) / 64; ++q) ss += red[q];
-    }
-    if (j < D) {
-      const float gv = ld_f32<T>(G, row * a.ld + hc + j);
-      const float gate = gv / (1.0f + expf(-gv));
-      st_f32<T>(Y, row * a.ldy + hc + j, o / sqrtf(ss / (float)D + a.eps) * nw * gate);
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+      const float v = mine ? sv[t][j] : 0.f;
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < DMAX; ++i) {
+        const float kv = sk[t][i] * v;
+        o += sr[t][i] * (S[i] + su[i] * kv);
+        S[i] = sw[t][i] * S[i] + kv;
+      }
+      // head RMS norm over the D outputs of this token, then channel weight and gate
+      float ss = wave_sum(live ? o * o : 0.f);
+      if (NWV > 1) {
+        __syncthreads();
+        if ((j & 63) == 0) red[j >> 6] = ss;
+        __syncthreads();
+        ss = 0.f;
+#pragma unroll
+        for (int q = 0; q < NWV; ++q) ss += red[q];
+      }
+      if (live) {
+        const float g = sg[t][j];
+        const float gate = g / (1.0f + expf(-g));
+        st_f32<T>(Y, (long)(base + t) * a.ldy + hc + j, o / sqrtf(ss * inv_d + a.eps) * nw * gate);
+      }
     }
   }
-  if (j < D) {
+  if (live) {
 #pragma unroll
     for (int i = 0; i < DMAX; ++i)
       if (i < D) Sg[(long)i * D + j] = S[i];

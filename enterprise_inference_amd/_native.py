@@ -70,7 +70,7 @@ _SIGNATURES = {
     "eia_latent_attn": [P, L, L, P, L, L, P, I, P, L, IP, I, IP, IP, IP, I, IP, P, L, P, L, L, F,
                         I, I, I, I, I, I, S],
     "eia_latent_attn_mfma": [P, L, L, P, L, L, P, I, P, L, IP, I, IP, IP, IP, I, IP, P, L, P, L, L,
-                             F, I, I, I, I, I, S],
+                             F, I, I, I, I, I, I, P, P, S],
     "eia_token_shift_mix": [P, P, I, P, IP, IP, I, IP, P, L, I, I, I, S],
     "eia_wkv_scan": [P, P, P, P, L, P, L, P, P, P, P, P, P, I, IP, IP, IP, IP, P, L, F, I, I, I,
                      I, S],

@@ -50,6 +50,21 @@ def query_block(num_heads: int, kv_rank: int, rot_dim: int = 0,
     return max(1, min(16, ACC_ROWS // (hb * kv_rank), 12288 // (hb * (kv_rank + rot_dim))))
 
 
+def decode_partitions(batch: int, num_heads: int, cus: int = 256) -> int:
+    """Key partitions (grid.z) of a decode launch of the MFMA form: a decode row is one
+    single-wave workgroup per 16-head slice, so small batches split every row's keys until about
+    four workgroups per CU exist (a power of two, at most 32); the partials are merged by a
+    second kernel.  Depends on the batch only, so a captured decode graph keeps its grid."""
+    forced = int(os.environ.get("EIA_LATENT_DECODE_P", "0"))
+    if forced > 0:
+        return min(forced, 64)
+    wgs = max(1, batch * ((num_heads + 15) // 16))
+    p = 1
+    while p < 32 and wgs * p * 2 <= 4 * cus:
+        p *= 2
+    return p
+
+
 def build_work(q_lens: List[int], qblock: int) -> List[int]:
     """[seq, first query] pairs, latest query blocks first (longest causal rows first)."""
     items = [(q0, s) for s, n in enumerate(q_lens) for q0 in range(0, n, qblock)]
@@ -183,12 +198,18 @@ def latent_attention(q_abs: torch.Tensor, q_rot: torch.Tensor, inv_freq: torch.T
         g = None if gate is None else gate[lo:]
         require(bt.dtype == torch.int32 and bt.stride(1) == 1, "block tables int32")
         if mfma:
+            P = decode_partitions(n_items, H) if cu is None else 1
+            pa = pm = None
+            if P > 1:
+                pa = torch.empty(n_items * H * P * R, dtype=torch.float32, device=q_abs.device)
+                pm = torch.empty(n_items * H * P * 2, dtype=torch.float32, device=q_abs.device)
             check(lib().eia_latent_attn_mfma(
                 ptr(qa), qa.stride(0), qa.stride(1), ptr(qr), qr.stride(0), qr.stride(1),
                 ptr(inv_freq), rot_dims, ptr(cache), cache.shape[-1], ptr(bt), bt.stride(0),
                 ptr(lens), ptr(cu), ptr(work), n_items, ptr(md.positions[lo:]), ptr(g),
                 g.stride(0) if g is not None else 0, ptr(o), o.stride(0), o.stride(1),
-                float(scale), H, R, rd, bs, qb, stream(q_abs)), "latent_attn_mfma")
+                float(scale), H, R, rd, bs, qb, P, ptr(pa), ptr(pm), stream(q_abs)),
+                "latent_attn_mfma")
             return
         check(lib().eia_latent_attn(
             ptr(qa), qa.stride(0), qa.stride(1), ptr(qr), qr.stride(0), qr.stride(1),

@@ -26,7 +26,7 @@ def test_kernel(case, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
-@pytest.mark.parametrize("shape", [(5, 24, 8), (20, 72, 16), (16, 264, 24), (2, 512, 64)],
+@pytest.mark.parametrize("shape", [(5, 24, 8), (20, 72, 16), (16, 256, 32), (16, 264, 24), (2, 512, 64)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_latent_attention_shapes(shape, dtype):
     """Head counts below, at and above a 16-head slice; latent widths of every MFMA variant
