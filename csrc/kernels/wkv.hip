@@ -74,21 +74,25 @@ struct WkvArgs {
   float eps; int H, D;
 };
 
-// One workgroup per (sequence, head); thread j owns column j of S (dk values in registers,
-// DMAX >= D) and walks the sequence's tokens in order.  Tokens are staged TC at a time: every
-// thread loads its channel of r, k, decay, v and the gate for TC tokens (coalesced over the
-// channels), r / k / w go to LDS, and the recurrence then runs TC steps on LDS broadcasts, so a
-// token costs one pass over dk instead of a global-memory round trip.
-#define WKV_TC (DMAX > 128 ? 8 : 16)
-
+// One workgroup per (sequence, head), 4 x max(64, DMAX) threads: thread (q, j) owns rows
+// [q DMAX/4, (q+1) DMAX/4) of column j of S in registers and walks the sequence's tokens in
+// order.  Tokens are staged TC at a time: r, k, decay, v and the gate of TC tokens go to LDS
+// (coalesced over the channels; channels >= D hold zeros so the dk loops run branch-free), the
+// recurrence runs TC steps on LDS broadcasts leaving four partial outputs per token and column,
+// and the partials are then summed, RMS-normed per head, weighted and gated -- so a token costs
+// a quarter pass over dk per thread instead of a global-memory round trip.
 template <typename T, int DMAX>
-__global__ void __launch_bounds__(DMAX < 64 ? 64 : DMAX)
+__global__ void __launch_bounds__(4 * (DMAX < 64 ? 64 : DMAX))
 wkv_scan_kernel(WkvArgs a) {
-  // channels >= D hold zeros, so the dk loops below run branch-free over DMAX
-  __shared__ __align__(16) float sr[WKV_TC][DMAX], sk[WKV_TC][DMAX], sw[WKV_TC][DMAX], su[DMAX];
-  __shared__ float sv[WKV_TC][DMAX], sg[WKV_TC][DMAX];
-  __shared__ float red[4];
-  const int s = blockIdx.x, h = blockIdx.y, j = threadIdx.x, D = a.D;
+  constexpr int DP = DMAX < 64 ? 64 : DMAX;          // threads per quarter
+  constexpr int DQ = DMAX / 4;                       // dk rows per thread
+  constexpr int TC = DMAX <= 64 ? 16 : DMAX <= 128 ? 8 : 4;
+  constexpr int NWV = DP / 64;                       // waves per quarter
+  __shared__ __align__(16) float sr[TC][DMAX], sk[TC][DMAX], sw[TC][DMAX], su[DMAX];
+  __shared__ float sv[TC][DMAX], sg[TC][DMAX], po[TC][4][DP];
+  __shared__ float red[4][NWV];
+  const int s = blockIdx.x, h = blockIdx.y, D = a.D;
+  const int q = threadIdx.x / DP, j = threadIdx.x % DP;
   const int slot = a.slots[s];
   if (slot < 0 || (a.seq_lens && a.seq_lens[s] <= 0)) return;
   const int lo = a.cu ? a.cu[s] : s, hi = a.cu ? a.cu[s + 1] : s + 1;
@@ -96,11 +100,13 @@ wkv_scan_kernel(WkvArgs a) {
   const bool fresh = a.positions[lo] == 0;
   const bool live = j < D, mine = j < DMAX;
   float* Sg = a.S + ((long)slot * a.H + h) * D * D;
-  float S[DMAX];
+  const int i0 = q * DQ;
+  float S[DQ];
 #pragma unroll
-  for (int i = 0; i < DMAX; ++i) S[i] = (!fresh && i < D && live) ? Sg[(long)i * D + j] : 0.f;
+  for (int i = 0; i < DQ; ++i)
+    S[i] = (!fresh && i0 + i < D && live) ? Sg[(long)(i0 + i) * D + j] : 0.f;
   const long hc = (long)h * D;
-  if (mine) su[j] = live ? ld_f32<T>(static_cast<const T*>(a.u), hc + j) : 0.f;
+  if (q == 0 && mine) su[j] = live ? ld_f32<T>(static_cast<const T*>(a.u), hc + j) : 0.f;
   const float w0 = live ? ld_f32<T>(static_cast<const T*>(a.w0), hc + j) : 0.f;
   const float nw = live ? ld_f32<T>(static_cast<const T*>(a.norm_w), hc + j) : 0.f;
   const T* R = static_cast<const T*>(a.r);
@@ -108,28 +114,30 @@ wkv_scan_kernel(WkvArgs a) {
   const T* V = static_cast<const T*>(a.v);
   const T* G = static_cast<const T*>(a.g);
   T* Y = static_cast<T*>(a.y);
-  constexpr int NWV = (DMAX + 63) / 64;
   const float inv_d = 1.0f / (float)D;
-  for (int base = lo; base < hi; base += WKV_TC) {
-    const int nt = min(WKV_TC, hi - base);
+  for (int base = lo; base < hi; base += TC) {
+    const int nt = min(TC, hi - base);
     __syncthreads();                       // the previous chunk's LDS reads are done
     if (mine) {
-#pragma unroll 4
-      for (int t = 0; t < nt; ++t) {
-        const long row = base + t;
-        float r = 0.f, k = 0.f, w = 0.f, v = 0.f, g = 0.f;
-        if (live) {
-          r = ld_f32<T>(R, row * a.ld + hc + j);
-          k = ld_f32<T>(K, row * a.ld + hc + j);
-          w = expf(-expf(a.dec[row * a.ld_dec + hc + j] + w0));
-          v = ld_f32<T>(V, row * a.ld + hc + j);
-          g = ld_f32<T>(G, row * a.ld + hc + j);
+#pragma unroll
+      for (int tt = 0; tt < TC / 4; ++tt) {            // quarter q stages tokens q, q + 4, ...
+        const int t = tt * 4 + q;
+        if (t < nt) {
+          const long row = base + t;
+          float r = 0.f, k = 0.f, w = 0.f, v = 0.f, g = 0.f;
+          if (live) {
+            r = ld_f32<T>(R, row * a.ld + hc + j);
+            k = ld_f32<T>(K, row * a.ld + hc + j);
+            w = expf(-expf(a.dec[row * a.ld_dec + hc + j] + w0));
+            v = ld_f32<T>(V, row * a.ld + hc + j);
+            g = ld_f32<T>(G, row * a.ld + hc + j);
+          }
+          sr[t][j] = r;
+          sk[t][j] = k;
+          sw[t][j] = w;
+          sv[t][j] = v;
+          sg[t][j] = g;
         }
-        sr[t][j] = r;
-        sk[t][j] = k;
-        sw[t][j] = w;
-        sv[t][j] = v;
-        sg[t][j] = g;
       }
     }
     __syncthreads();
@@ -137,22 +145,30 @@ wkv_scan_kernel(WkvArgs a) {
       const float v = mine ? sv[t][j] : 0.f;
       float o = 0.f;
 #pragma unroll
-      for (int i = 0; i < DMAX; ++i) {
-        const float kv = sk[t][i] * v;
-        o += sr[t][i] * (S[i] + su[i] * kv);
-        S[i] = sw[t][i] * S[i] + kv;
+      for (int i = 0; i < DQ; ++i) {
+        const float kv = sk[t][i0 + i] * v;
+        o += sr[t][i0 + i] * (S[i] + su[i0 + i] * kv);
+        S[i] = sw[t][i0 + i] * S[i] + kv;
       }
-      // head RMS norm over the D outputs of this token, then channel weight and gate
-      float ss = wave_sum(live ? o * o : 0.f);
+      po[t][q][j] = o;
+    }
+    __syncthreads();
+    // quarter q finishes tokens q, q + 4, ...: sum of the partials, head RMS norm, weight, gate
+#pragma unroll
+    for (int tt = 0; tt < TC / 4; ++tt) {
+      const int t = tt * 4 + q;
+      const bool ok = t < nt && live;
+      const float o = ok ? po[t][0][j] + po[t][1][j] + po[t][2][j] + po[t][3][j] : 0.f;
+      float ss = wave_sum(o * o);
       if (NWV > 1) {
         __syncthreads();
-        if ((j & 63) == 0) red[j >> 6] = ss;
+        if ((j & 63) == 0) red[q][j >> 6] = ss;
         __syncthreads();
         ss = 0.f;
 #pragma unroll
-        for (int q = 0; q < NWV; ++q) ss += red[q];
+        for (int x = 0; x < NWV; ++x) ss += red[q][x];
       }
-      if (live) {
+      if (ok) {
         const float g = sg[t][j];
         const float gate = g / (1.0f + expf(-g));
         st_f32<T>(Y, (long)(base + t) * a.ldy + hc + j, o / sqrtf(ss * inv_d + a.eps) * nw * gate);
@@ -161,13 +177,13 @@ wkv_scan_kernel(WkvArgs a) {
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i)
-      if (i < D) Sg[(long)i * D + j] = S[i];
+    for (int i = 0; i < DQ; ++i)
+      if (i0 + i < D) Sg[(long)(i0 + i) * D + j] = S[i];
   }
   if (h == 0) {
     const float* last = a.x + (long)(hi - 1) * a.W;
     float* p = a.prev + (long)slot * a.W;
-    for (int c = j; c < a.W; c += blockDim.x) p[c] = last[c];
+    for (int c = threadIdx.x; c < a.W; c += blockDim.x) p[c] = last[c];
   }
 }
 
@@ -184,7 +200,7 @@ EIA_API int eia_wkv_scan(const void* r, const void* k, const void* v, const void
             seq_lens, y, ldy, eps, H, D};
   dim3 grid(nseq, H);
 #define WKV_LAUNCH(TT, DM)                                                                 \
-  hipLaunchKernelGGL((wkv_scan_kernel<TT, DM>), grid, dim3(DM < 64 ? 64 : DM), 0, st, a)
+  hipLaunchKernelGGL((wkv_scan_kernel<TT, DM>), grid, dim3(4 * (DM < 64 ? 64 : DM)), 0, st, a)
   if (is_bf16) {
     if (D <= 32) WKV_LAUNCH(bf16_t, 32);
     else if (D <= 64) WKV_LAUNCH(bf16_t, 64);
