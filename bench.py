@@ -67,7 +67,7 @@ def parse():
     ap.add_argument("--mode", default="endpoint", choices=["endpoint", "engine", "design"],
                     help="design: prefill / decode throughput of the Sekolorn design beside a "
                          "Mixtral-style decoder at equal layer sizes (benchmarks/design_bench.py)")
-    ap.add_argument("--design-sizes", default="s,m", help="comma list of s, m, l")
+    ap.add_argument("--design-sizes", default="s,s6", help="comma list of s, s6 (m, l: gated)")
     ap.add_argument("--design-models", default="sekolorn,mixtral",
                     help="which of the two engines to run (profiling one of them alone)")
     ap.add_argument("--design-kernels", action="store_true",

@@ -23,11 +23,18 @@ SIZES = {
     #       experts, top, groups, keep, ff, vocab
     "s": dict(width=1024, layers=3, heads=8, dim=64, rot=32, kv_rank=128, q_rank=256,
               wkv_heads=16, experts=8, top=2, groups=4, keep=2, ff=512, vocab=32000),
+    "s6": dict(width=1024, layers=6, heads=8, dim=64, rot=32, kv_rank=128, q_rank=256,
+               wkv_heads=16, experts=8, top=2, groups=4, keep=2, ff=512, vocab=32000),
     "m": dict(width=2048, layers=6, heads=16, dim=64, rot=32, kv_rank=256, q_rank=512,
               wkv_heads=32, experts=16, top=2, groups=4, keep=2, ff=1024, vocab=32000),
     "l": dict(width=4096, layers=6, heads=32, dim=128, rot=64, kv_rank=512, q_rank=1536,
               wkv_heads=64, experts=16, top=4, groups=4, keep=2, ff=1536, vocab=32000),
 }
+# Sizes whose whole-engine run is switched off on the GPU: a profiled run of the two "m"
+# engines ended with a GPU fault whose cause was not found (every kernel variant those sizes
+# select passes its unit tests, the engines were never seen to fail unprofiled); they raise
+# until that cause is shown.
+GATED = {"m", "l"}
 
 
 def sekolorn_config(z: dict) -> dict:
@@ -113,6 +120,9 @@ def _measure(cfg_dict: dict, a) -> dict:
 def run(a) -> int:
     rows = []
     for name in a.design_sizes.split(","):
+        if name in GATED:
+            raise SystemExit(f"design size {name!r} is switched off (see GATED in "
+                             "benchmarks/design_bench.py); run s or s6")
         z = SIZES[name]
         for label, cfg in (("Sekolorn", sekolorn_config(z)), ("Mixtral-style", mixtral_config(z))):
             if label.split("-")[0].lower() not in a.design_models.lower():
