@@ -606,3 +606,59 @@ EIA_API int eia_moe_route_grouped(const void* x, long ldx, const void* wr, int H
                        (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len);
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// End of an expert block with a post-norm on an fp32 residual stream, one launch per step:
+//   y = sum_s w[t][s] * h2[inv[t][s]]  (+ shared[t]);   x[t] += layernorm(y) * nw;   xb[t] = (T) x[t]
+// (layer norm with a weight and no bias; the expert sum, the norm and the residual are fp32).
+// One workgroup per token; the row is kept in LDS between the passes.
+template <typename T>
+__global__ void __launch_bounds__(256)
+combine_postnorm_kernel(const T* __restrict__ h2, long ldh, const float* __restrict__ w,
+                        const int* __restrict__ inv, int k, const T* __restrict__ shared,
+                        long lds_, const T* __restrict__ nw, float eps, float* __restrict__ x,
+                        T* __restrict__ xb, long ldxb, int W) {
+  extern __shared__ float rowbuf[];
+  __shared__ float scratch[4];
+  const long t = blockIdx.x;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float y = shared ? ld_f32<T>(shared, t * lds_ + c) : 0.f;
+    for (int j = 0; j < k; ++j) {
+      const int pos = inv[t * k + j];
+      if (pos >= 0) y += w[t * k + j] * ld_f32<T>(h2, (long)pos * ldh + c);
+    }
+    rowbuf[c] = y;
+    s += y;
+  }
+  const float mean = block_sum(s, scratch) / (float)W;
+  float q = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float d = rowbuf[c] - mean;
+    q += d * d;
+  }
+  const float is = 1.0f / sqrtf(block_sum(q, scratch) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = x[t * W + c] + (rowbuf[c] - mean) * is * ld_f32<T>(nw, c);
+    x[t * W + c] = v;
+    if (xb) st_f32<T>(xb + t * ldxb, c, v);
+  }
+}
+
+EIA_API int eia_moe_combine_postnorm(const void* h2, long ldh, const float* w, const int* inv,
+                                     int k, const void* shared, long lds_, const void* nw,
+                                     float eps, float* x, void* xb, long ldxb, int T, int W,
+                                     int is_bf16, hipStream_t st) {
+  if (T < 0 || W < 1 || k < 1 || W > 16384) return EIA_BAD_SHAPE;
+  if (T == 0) return EIA_OK;
+  const size_t lds = (size_t)W * 4;
+  if (is_bf16)
+    hipLaunchKernelGGL((combine_postnorm_kernel<bf16_t>), dim3(T), dim3(256), lds, st,
+                       (const bf16_t*)h2, ldh, w, inv, k, (const bf16_t*)shared, lds_,
+                       (const bf16_t*)nw, eps, x, (bf16_t*)xb, ldxb, W);
+  else
+    hipLaunchKernelGGL((combine_postnorm_kernel<float>), dim3(T), dim3(256), lds, st,
+                       (const float*)h2, ldh, w, inv, k, (const float*)shared, lds_,
+                       (const float*)nw, eps, x, (float*)xb, ldxb, W);
+  EIA_LAUNCH_CHECK();
+}

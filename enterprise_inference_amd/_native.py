@@ -76,6 +76,7 @@ _SIGNATURES = {
                      I, S],
     "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, S],
     "eia_relu2": [P, P, L, I, S],
+    "eia_moe_combine_postnorm": [P, L, P, P, I, P, L, P, F, P, P, L, I, I, I, S],
     "eia_ar_alloc": [P, L],
     "eia_moe_splitk_norm_route": [P, I, I, I, P, P, F, P, L, P, I, I, I, I, P, P, P, S],
     "eia_moe_combine_norm": [P, I, I, P, P, I, I, I, P, P, F, P, L, S],

@@ -233,16 +233,32 @@ class GroupRoutedMoE(nn.Module):
             lambda p, t, sid=None: p.data[sid].copy_(t)
         self.shared = UngatedMLP(hidden, shared_inter, dtype, device) if shared_inter else None
 
-    def forward(self, x, md=None):
+    def _route(self, x, md):
         row_len = None
         if md is not None and md.num_prefill_tokens == 0 and md.decode_seq_lens is not None:
             row_len = md.decode_seq_lens          # bucket-padding rows route nowhere
-        tw, ids = moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
-                                        self.route_scale, row_len)
+        return moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
+                                     self.route_scale, row_len)
+
+    def forward(self, x, md=None):
+        tw, ids = self._route(x, md)
         out = moe_ops.ungated_moe(x, self.w_up, self.w_down, tw, ids, "relu2")
         if self.shared is not None:
             out = out + self.shared(x)
         return out
+
+    def forward_post_norm(self, x, md, norm_w, eps: float, resid: torch.Tensor):
+        """resid += layernorm(block(x)) * norm_w (fp32, in place); returns resid in x's dtype.
+        On the GPU the experts' weighted sum, the shared expert's add, the norm and the
+        residual update are one launch."""
+        from ..ops import norm as norm_ops
+        if not x.is_cuda:
+            return norm_ops.post_norm_residual(self.forward(x, md), norm_w, eps, resid)
+        tw, ids = self._route(x, md)
+        h2, inv = moe_ops.ungated_moe(x, self.w_up, self.w_down, tw, ids, "relu2",
+                                      rows_only=True)
+        shared = self.shared(x) if self.shared is not None else None
+        return moe_ops.combine_post_norm(h2, tw, inv, shared, norm_w, eps, resid)
 
 
 class MixtralForCausalLM(LlamaForCausalLM):

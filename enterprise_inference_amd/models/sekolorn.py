@@ -73,7 +73,7 @@ class SekolornLayer(nn.Module):
         y = self.mix(x, md, cache) if self.kind == "wkv" else self.mix(xb, md, cache)
         xb = norm_ops.post_norm_residual(y, self.norm1, self.eps, x)
         if self.mlp is not None:
-            xb = norm_ops.post_norm_residual(self.mlp(xb, md), self.norm2, self.eps, x)
+            xb = self.mlp.forward_post_norm(xb, md, self.norm2, self.eps, x)
         return xb
 
 

@@ -364,8 +364,11 @@ def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: i
 
 
 def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_w: torch.Tensor,
-                topk_ids: torch.Tensor, act: str = "relu2") -> torch.Tensor:
+                topk_ids: torch.Tensor, act: str = "relu2", rows_only: bool = False):
     """Experts without a gate branch: y = sum_k w_k * W_down[e_k] act(W_up[e_k] x).
+    ``rows_only`` (GPU): return (expert output rows in sorted order [T*k, H], inv int32 [T*k]
+    mapping (token, choice) to its row, -1 for no expert) and leave the weighted sum to the
+    caller (``combine_post_norm``).
     x [T, H]; w_up [E, I, H]; w_down [E, H, I] -> [T, H].  Rows are sorted by expert on the
     device (moe.hip align), the E+1 offsets are read back once, and each expert runs one library
     GEMM pair on its contiguous slice; one activation launch covers all slices.  An id >= E
@@ -409,6 +412,8 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
         check(lib().eia_moe_gemm(ptr(h1), h1.stride(0), ptr(w_down), w_down.stride(1), None,
                                  ptr(h2), h2.stride(0), H, I, E, ptr(offs), None, mt, 0,
                                  2 if H % 128 == 0 else 0, st), "moe_gemm_down")
+        if rows_only:
+            return h2, inv
         out = torch.empty(T, H, dtype=x.dtype, device=dev)
         check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
                                     ptr(out), out.stride(0), st), "moe_combine")
@@ -423,6 +428,8 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
         check(lib().eia_moe_grouped_gemm(ptr(h1), h1.stride(0), None, ptr(w_down), H, I, E,
                                          ptr(offs), n, 0, ptr(h2), h2.stride(0), st),
               "moe_grouped_gemm_down")
+        if rows_only:
+            return h2, inv
         out = torch.empty(T, H, dtype=x.dtype, device=dev)
         check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
                                     ptr(out), out.stride(0), st), "moe_combine")
@@ -444,6 +451,8 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
         a, b = bounds[e], bounds[e + 1]
         if a < b:
             torch.matmul(h1[a:b], w_down[e].t(), out=h2[a:b])
+    if rows_only:
+        return h2, inv
     if x.dtype == torch.bfloat16 and H % 8 == 0:
         out = torch.empty(T, H, dtype=x.dtype, device=dev)
         check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
@@ -451,3 +460,26 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
         return out
     rows = h2.index_select(0, inv[:n].long().clamp_(0, max(0, n - 1))).view(T, k, H)
     return (rows.float() * topk_w[:, :, None]).sum(1).to(x.dtype)
+
+
+def combine_post_norm(h2: torch.Tensor, topk_w: torch.Tensor, inv: torch.Tensor,
+                      shared: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                      x: torch.Tensor, copy: bool = True) -> Optional[torch.Tensor]:
+    """End of an expert block under a post-norm (moe.hip combine_postnorm_kernel, one launch):
+    y = sum_s w[t, s] h2[inv[t, s]] (+ shared[t]);  x += layernorm(y) * norm_w in place (fp32);
+    returns the new x in h2's dtype (an fp32 model gets x itself)."""
+    T, k = topk_w.shape
+    W = x.shape[1]
+    bf = h2.dtype == torch.bfloat16
+    require(h2.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and
+            h2.stride(1) == 1 and (bf or h2.dtype == torch.float32) and norm_w.dtype == h2.dtype
+            and inv.dtype == torch.int32 and topk_w.dtype == torch.float32 and W <= 16384,
+            "combine_post_norm: layout")
+    require(shared is None or (shared.dtype == h2.dtype and shared.stride(1) == 1 and
+                               shared.shape == (T, W)), "combine_post_norm: shared rows")
+    xb = torch.empty(T, W, dtype=h2.dtype, device=h2.device) if (copy and bf) else None
+    check(lib().eia_moe_combine_postnorm(
+        ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), k, ptr(shared),
+        shared.stride(0) if shared is not None else 0, ptr(norm_w), float(eps), ptr(x), ptr(xb),
+        W, T, W, 1 if bf else 0, stream(h2)), "moe_combine_postnorm")
+    return xb if bf else (x if copy else None)

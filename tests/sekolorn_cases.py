@@ -114,6 +114,36 @@ def case_ungated_moe(device, dtype, E=5, I=12, H=24, T=11, k=2):
         assert torch.allclose(out[t].double(), want, atol=ktol(dtype) * 4, rtol=ktol(dtype) * 4)
 
 
+def case_combine_post_norm(device, dtype):
+    """Fused end of the expert block: weighted sum of expert rows (+ shared rows), layer norm,
+    add to the fp32 residual, copy in the activation type."""
+    from enterprise_inference_amd.ops import moe
+    g = torch.Generator().manual_seed(8)
+    for T, k, W, with_shared in ((7, 2, 40, True), (3, 3, 256, False), (5, 1, 1030, True)):
+        n = T * k
+        h2 = torch.randn(n, W, generator=g).to(dtype)
+        inv = torch.randperm(n, generator=g).to(torch.int32).view(T, k)
+        tw = torch.rand(T, k, generator=g)
+        inv[1, k - 1] = -1                                   # a choice that routed nowhere
+        shared = torch.randn(T, W, generator=g).to(dtype) if with_shared else None
+        nw = (1 + 0.3 * torch.randn(W, generator=g)).to(dtype)
+        x = torch.randn(T, W, generator=g)
+        y = torch.zeros(T, W, dtype=torch.float64)
+        for t in range(T):
+            for s_ in range(k):
+                if inv[t, s_] >= 0:
+                    y[t] += float(tw[t, s_]) * h2[int(inv[t, s_])].double()
+            if shared is not None:
+                y[t] += shared[t].double()
+        want = x.double() + O.layer_norm_nobias(y, nw.double(), 1e-5)
+        xd = x.clone().to(device)
+        xb = moe.combine_post_norm(h2.to(device), tw.to(device), inv.view(-1).to(device),
+                                   None if shared is None else shared.to(device), nw.to(device),
+                                   1e-5, xd)
+        assert torch.allclose(xd.cpu().double(), want, atol=2e-5, rtol=2e-5), (T, k, W)
+        assert torch.allclose(xb.float().cpu(), xd.cpu().to(dtype).float())
+
+
 def _paged(rows_c, rows_kr, block_size, nblocks, order, dtype, device):
     """Scatter cache rows of one sequence into a paged cache using block list ``order``."""
     n, R = rows_c.shape

@@ -18,7 +18,7 @@ def _cfg(fn, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 @pytest.mark.parametrize("case", [K.case_post_norm, K.case_route, K.case_route_group_limit,
-                                  K.case_ungated_moe, K.case_latent_prep,
+                                  K.case_ungated_moe, K.case_combine_post_norm, K.case_latent_prep,
                                   K.case_latent_attention_needle, K.case_wkv],
                          ids=lambda f: f.__name__)
 def test_kernel(case, dtype):
