@@ -73,6 +73,45 @@ def config_c():
             ]}
 
 
+def config_d():
+    """Sizes that are multiples of nothing: width 100, 5 heads of 10 + 6, latent 36, 9 experts in
+    3 groups with top 4, wkv head size 24; three latent layers sharing one cache, the owner
+    first."""
+    return {"architecture": "Sekolorn", "vocab": 130, "width": 100, "norm": {"eps": 1e-5},
+            "layers": [
+                {"type": "latent_attention",
+                 "mixer": latent(heads=5, dim=10, rot_dim=6, vdim=14, kv_rank=36, q_rank=22,
+                                 scale=0.3, rot_dims=6, base=1000.0),
+                 "mlp": moe(experts=9, top=4, count=3, keep=2, ff=20, shared=12, scale=0.9)},
+                {"type": "latent_attention",
+                 "mixer": latent(heads=2, dim=18, rot_dim=6, vdim=6, kv_rank=36, q_rank=30,
+                                 scale=0.25, rot_dims=6, base=1000.0, kv_from=0), "mlp": None},
+                {"type": "wkv", "mixer": {"heads": 2, "dim": 24, "decay_rank": 5},
+                 "mlp": moe(experts=2, top=1, count=2, keep=2, ff=28, shared=0)},
+                {"type": "latent_attention",
+                 "mixer": latent(heads=3, dim=12, rot_dim=6, vdim=12, kv_rank=36, q_rank=16,
+                                 scale=0.3, rot_dims=6, base=1000.0, kv_from=0),
+                 "mlp": moe(experts=3, top=3, count=1, keep=1, ff=12, shared=100)},
+            ]}
+
+
+def config_e():
+    """Layer shapes of a mid-size model at a small width: 16 heads on a 256-wide latent with a
+    32-wide rotary part, 16 experts in 4 groups, wkv heads of 64; graph-eligible."""
+    return {"architecture": "Sekolorn", "vocab": 200, "width": 128, "norm": {"eps": 1e-6},
+            "layers": [
+                {"type": "latent_attention",
+                 "mixer": latent(heads=16, dim=16, rot_dim=32, vdim=16, kv_rank=256, q_rank=64,
+                                 scale=0.15, base=10000.0),
+                 "mlp": moe(experts=16, top=2, count=4, keep=2, ff=128, shared=128)},
+                {"type": "wkv", "mixer": {"heads": 4, "dim": 64, "decay_rank": 16},
+                 "mlp": moe(experts=16, top=2, count=4, keep=2, ff=128, shared=0)},
+                {"type": "latent_attention",
+                 "mixer": latent(heads=16, dim=16, rot_dim=32, vdim=16, kv_rank=256, q_rank=64,
+                                 scale=0.15, base=10000.0, kv_from=0), "mlp": None},
+            ]}
+
+
 def all_experts(cfg: dict) -> dict:
     """The same model with every expert of every group chosen.  With bf16 activations a
     router score that nearly ties another can pick a different expert than the float64 oracle

@@ -31,6 +31,10 @@ def test_schedules_config_b():
     K.case_schedules(DEV, DT, C.config_b, seed=7)
 
 
+def test_schedules_config_d():
+    K.case_schedules(DEV, DT, C.config_d, seed=11)
+
+
 def test_long_decode():
     K.case_long_decode(DEV, DT)
 

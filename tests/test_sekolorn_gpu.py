@@ -54,6 +54,20 @@ def test_schedules_config_b(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_schedules_config_d(dtype):
+    K.case_schedules("cuda", dtype, _cfg(C.config_d, dtype), seed=11)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
+def test_schedules_config_e(dtype):
+    K.case_schedules("cuda", dtype, _cfg(C.config_e, dtype), seed=13)
+
+
+def test_generate_graph_decode_config_e():
+    K.case_generate("cuda", torch.bfloat16, _cfg(C.config_e, torch.bfloat16), expect_graphs=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
 def test_long_decode(dtype):
     K.case_long_decode("cuda", dtype, _cfg(C.config_b, dtype))
 
