@@ -543,12 +543,19 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
   const int t = blockIdx.x * 4 + wave;
   if (t >= T_) return;
   const T* xr = x + (long)t * ldx;
-  for (int e = 0; e < E; ++e) {
-    const T* w = wr + (long)e * H;
-    float p = 0.f;
-    for (int c = lane; c < H; c += 64) p += ld_f32<T>(xr, c) * ld_f32<T>(w, c);
-    p = wave_sum(p);
-    if (lane == 0) sc[wave][e] = 1.0f / (1.0f + expf(-p));
+  for (int e0 = 0; e0 < E; e0 += 8) {          // eight experts per pass over the token's row
+    float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int c = lane; c < H; c += 64) {
+      const float xv = ld_f32<T>(xr, c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (e0 + j < E) p[j] += xv * ld_f32<T>(wr, (long)(e0 + j) * H + c);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float v = wave_sum(p[j]);
+      if (lane == 0 && e0 + j < E) sc[wave][e0 + j] = 1.0f / (1.0f + expf(-v));
+    }
   }
   if (lane != 0) return;
   float* s = sc[wave];

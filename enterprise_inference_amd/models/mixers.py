@@ -13,8 +13,6 @@ returns the mixer output in the activation dtype.
 
 from __future__ import annotations
 
-from typing import Optional
-
 import torch
 import torch.nn as nn
 

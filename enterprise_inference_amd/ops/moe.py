@@ -328,6 +328,9 @@ def _fused_moe_per_expert(x, w13, w2, topk_w, topk_ids, e_lo, act):
 
 
 UNGATED_GROUPED = os.environ.get("EIA_UNGATED_GROUPED", "1") != "0"
+# experts up to this many weights per matrix stay on the grouped MFMA kernel at any row count:
+# their per-expert library GEMMs are launch- and read-back-bound, not MFMA-bound
+UNGATED_SMALL_EXPERT = int(os.environ.get("EIA_UNGATED_SMALL_EXPERT", str(2 * 1024 * 1024)))
 
 
 def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: int,
@@ -418,8 +421,8 @@ def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_
         check(lib().eia_moe_combine(ptr(h2), h2.stride(0), ptr(topk_w), ptr(inv), T, k, H,
                                     ptr(out), out.stride(0), st), "moe_combine")
         return out
-    if bf and H % 128 == 0 and I % 128 == 0 and (avg <= MFMA_MAX_ROWS or capturing) \
-            and UNGATED_GROUPED:
+    if bf and H % 128 == 0 and I % 128 == 0 and UNGATED_GROUPED and (
+            avg <= MFMA_MAX_ROWS or capturing or I * H <= UNGATED_SMALL_EXPERT):
         h1 = torch.empty(max(1, n), I, dtype=x.dtype, device=dev)
         h2 = torch.empty(max(1, n), H, dtype=x.dtype, device=dev)
         check(lib().eia_moe_grouped_gemm(ptr(x), x.stride(0), ptr(row_idx), ptr(w_up), I, H, E,
