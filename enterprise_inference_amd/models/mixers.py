@@ -64,7 +64,11 @@ class LatentAttentionMixer(nn.Module):
         # one fused down-projection of the layer input: [query latent | KV latent | shared rotary
         # key | head gates]; a layer reading another layer's cache has no KV rows
         self.kv_rows = kv_rank + rot_dim if own_kv else 0
-        self.down = _param((q_rank + self.kv_rows + heads, width), dtype, device)
+        # (rows padded with zeros to a multiple of 64: decode-sized batches then run the
+        # weight-streaming GEMM, whose row tiles need it; the pad columns are never read)
+        n = q_rank + self.kv_rows + heads
+        self.down = _param((-(-n // 64) * 64, width), dtype, device)
+        self.down.data[n:].zero_()
         self.down.weight_loader = self._load_down
         self.q_norm = _plain((q_rank,), dtype, device)
         self.kv_norm = _plain((kv_rank,), dtype, device) if own_kv else None
@@ -93,7 +97,8 @@ class LatentAttentionMixer(nn.Module):
         q = gemm.linear(cq, self.uq).view(T, H, D + rd)
         # key up-projection folded into the query: q_abs[t, h] = W_uk[h]^T q_nope[t, h]
         q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk.view(H, D, R)).transpose(0, 1)
-        gate = fused[:, self.q_rank + self.kv_rows:]
+        g0 = self.q_rank + self.kv_rows
+        gate = fused[:, g0:g0 + H]
         lat = lat_ops.latent_attention(q_abs, q[:, :, D:], self.inv_freq, self.rot_dims,
                                        cache.rows, md, gate, self.scale)
         # value up-projection of the attended latent, heads concatenated
