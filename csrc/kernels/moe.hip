@@ -530,32 +530,105 @@ EIA_API int eia_moe_combine_sk(const float* part, int sk, int rows, const float*
 // form `ngroups` equal groups of neighbours, a group scores the sum of its two largest s, only
 // experts of the `keep` best groups are eligible, the `k` largest eligible scores win and weigh
 // s * route_scale (not renormalised).  Ties go to the lower index.  One wave per token: lanes
-// split the width for the dot products, lane 0 selects (E <= 256).
+// split the width for the dot products; up to 64 experts the lanes then rank themselves with
+// shuffles (lane e = expert e), above that lane 0 selects serially (E <= 256).
 template <typename T>
 __global__ void __launch_bounds__(256)
 route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr, int H, int T_,
                      int E, int k, int ngroups, int keep, float route_scale,
                      float* __restrict__ tw, int* __restrict__ ids,
-                     const int* __restrict__ row_len) {
+                     const int* __restrict__ row_len, int extra) {
+  // extra = 1: one more output column per token naming expert E with weight 1 (an always-on
+  // expert stored behind the routed ones); "nowhere" is then E + 1
+  const int ko = k + extra, none = E + extra;
   __shared__ float sc[4][256];
   __shared__ unsigned char ok[4][256];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T_) return;
   const T* xr = x + (long)t * ldx;
+  float mine = -1.f;                           // lane e keeps expert e's score (E <= 64)
+  const bool vec8 = (H & 7) == 0 && (ldx & 7) == 0;
   for (int e0 = 0; e0 < E; e0 += 8) {          // eight experts per pass over the token's row
     float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int c = lane; c < H; c += 64) {
-      const float xv = ld_f32<T>(xr, c);
+    if constexpr (sizeof(T) == 2) {
+      if (vec8) {                              // 16-byte loads: 8 consecutive channels per lane
+        for (int c = lane * 8; c < H; c += 512) {
+          const bf16x8 xv = *reinterpret_cast<const bf16x8*>(xr + c);
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if (e0 + j < E) p[j] += xv * ld_f32<T>(wr, (long)(e0 + j) * H + c);
+          for (int j = 0; j < 8; ++j) {
+            if (e0 + j < E) {
+              const bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + (long)(e0 + j) * H + c);
+#pragma unroll
+              for (int q = 0; q < 8; ++q) p[j] += bf2f(xv[q]) * bf2f(wv[q]);
+            }
+          }
+        }
+      }
+    }
+    if (!(sizeof(T) == 2 && vec8)) {
+      for (int c = lane; c < H; c += 64) {
+        const float xv = ld_f32<T>(xr, c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (e0 + j < E) p[j] += xv * ld_f32<T>(wr, (long)(e0 + j) * H + c);
+      }
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float v = wave_sum(p[j]);
-      if (lane == 0 && e0 + j < E) sc[wave][e0 + j] = 1.0f / (1.0f + expf(-v));
+      const float v = wave_sum(p[j]);             // every lane holds the total
+      if (e0 + j < E) {
+        const float sg = 1.0f / (1.0f + expf(-v));
+        if (lane == 0) sc[wave][e0 + j] = sg;
+        if (lane == e0 + j) mine = sg;
+      }
     }
+  }
+  if (E <= 64) {
+    // lane e = expert e: ranks by counting better lanes (ties to the lower index), no LDS
+    const bool pad = row_len && row_len[t] == 0;
+    const int per = E / ngroups;
+    const bool real = lane < E;
+    const int grp = real ? lane / per : -1;
+    int r = 0;
+    for (int o = 0; o < E; ++o) {
+      const float so = __shfl(mine, o, 64);
+      if (real && o / per == grp && (so > mine || (so == mine && o < lane))) ++r;
+    }
+    const float contrib = (real && r < 2) ? mine : 0.f;
+    float gsum = 0.f;
+    for (int o = 0; o < E; ++o) {
+      const float co = __shfl(contrib, o, 64);
+      if (o / per == grp) gsum += co;
+    }
+    int grank = 0;
+    for (int g2 = 0; g2 < ngroups; ++g2) {
+      const float go = __shfl(gsum, g2 * per, 64);
+      if (real && (go > gsum || (go == gsum && g2 < grp))) ++grank;
+    }
+    const bool elig = real && grank < keep;
+    int fr = 0;
+    for (int o = 0; o < E; ++o) {
+      const float so = __shfl(mine, o, 64);
+      const int eo = __shfl((int)elig, o, 64);
+      if (eo && (so > mine || (so == mine && o < lane))) ++fr;
+    }
+    if (pad) {
+      if (lane < ko) {
+        ids[(long)t * ko + lane] = none;
+        tw[(long)t * ko + lane] = 0.f;
+      }
+    } else {
+      if (elig && fr < k) {
+        ids[(long)t * ko + fr] = lane;
+        tw[(long)t * ko + fr] = mine * route_scale;
+      }
+      if (extra && lane == 0) {
+        ids[(long)t * ko + k] = E;
+        tw[(long)t * ko + k] = 1.f;
+      }
+    }
+    return;
   }
   if (lane != 0) return;
   float* s = sc[wave];
@@ -586,31 +659,38 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
     for (int e = 0; e < E; ++e)
       if (el[e] == 1 && (best < 0 || s[e] > bv)) { best = e; bv = s[e]; }
     if (best < 0 || pad) {
-      ids[(long)t * k + r] = E;             // routes nowhere
-      tw[(long)t * k + r] = 0.f;
+      ids[(long)t * ko + r] = none;         // routes nowhere
+      tw[(long)t * ko + r] = 0.f;
     } else {
       el[best] = 2;
-      ids[(long)t * k + r] = best;
-      tw[(long)t * k + r] = bv * route_scale;
+      ids[(long)t * ko + r] = best;
+      tw[(long)t * ko + r] = bv * route_scale;
     }
+  }
+  if (extra) {
+    ids[(long)t * ko + k] = pad ? none : E;
+    tw[(long)t * ko + k] = pad ? 0.f : 1.f;
   }
 }
 
 // x [T, H] (row stride ldx) and wr [E, H] in bf16 (is_bf16) or fp32 -> tw fp32 [T, k], ids [T, k].
 EIA_API int eia_moe_route_grouped(const void* x, long ldx, const void* wr, int H, int T, int E,
                                   int k, int ngroups, int keep, float route_scale, float* tw,
-                                  int* ids, const int* row_len, int is_bf16, hipStream_t st) {
+                                  int* ids, const int* row_len, int extra, int is_bf16,
+                                  hipStream_t st) {
   if (E < 1 || E > 256 || k < 1 || ngroups < 1 || E % ngroups || keep < 1 || keep > ngroups ||
-      k > keep * (E / ngroups))
+      k > keep * (E / ngroups) || (extra != 0 && extra != 1))
     return EIA_BAD_SHAPE;
   if (T <= 0) return EIA_OK;
   dim3 grid((T + 3) / 4), block(256);
   if (is_bf16)
     hipLaunchKernelGGL((route_grouped_kernel<bf16_t>), grid, block, 0, st, (const bf16_t*)x, ldx,
-                       (const bf16_t*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len);
+                       (const bf16_t*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
+                       extra);
   else
     hipLaunchKernelGGL((route_grouped_kernel<float>), grid, block, 0, st, (const float*)x, ldx,
-                       (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len);
+                       (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
+                       extra);
   EIA_LAUNCH_CHECK();
 }
 

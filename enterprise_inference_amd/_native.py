@@ -74,7 +74,7 @@ _SIGNATURES = {
     "eia_token_shift_mix": [P, P, I, P, IP, IP, I, IP, P, L, I, I, I, S],
     "eia_wkv_scan": [P, P, P, P, L, P, L, P, P, P, P, P, P, I, IP, IP, IP, IP, P, L, F, I, I, I,
                      I, S],
-    "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, S],
+    "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, I, S],
     "eia_relu2": [P, P, L, I, S],
     "eia_moe_combine_postnorm": [P, L, P, P, I, P, L, P, F, P, P, L, I, I, I, S],
     "eia_ar_alloc": [P, L],

@@ -226,19 +226,24 @@ class GroupRoutedMoE(nn.Module):
         self.E, self.k, self.groups, self.keep = num_experts, top_k, num_groups, keep_groups
         self.route_scale = float(route_scale)
         self.router = _param((num_experts, hidden), dtype, device)
-        self.w_up = _param((num_experts, inter, hidden), dtype, device)
-        self.w_down = _param((num_experts, hidden, inter), dtype, device)
+        # a shared expert of the routed experts' size is stored as expert E and named by an extra
+        # routing column of weight 1: it then rides in the routed experts' grouped launches
+        self.merged_shared = shared_inter == inter and shared_inter > 0
+        n = num_experts + (1 if self.merged_shared else 0)
+        self.w_up = _param((n, inter, hidden), dtype, device)
+        self.w_down = _param((n, hidden, inter), dtype, device)
         self.router.weight_loader = lambda p, t, sid=None: p.data.copy_(t)
         self.w_up.weight_loader = self.w_down.weight_loader = \
             lambda p, t, sid=None: p.data[sid].copy_(t)
-        self.shared = UngatedMLP(hidden, shared_inter, dtype, device) if shared_inter else None
+        self.shared = UngatedMLP(hidden, shared_inter, dtype, device) \
+            if (shared_inter and not self.merged_shared) else None
 
     def _route(self, x, md):
         row_len = None
         if md is not None and md.num_prefill_tokens == 0 and md.decode_seq_lens is not None:
             row_len = md.decode_seq_lens          # bucket-padding rows route nowhere
         return moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
-                                     self.route_scale, row_len)
+                                     self.route_scale, row_len, always_on=self.merged_shared)
 
     def forward(self, x, md=None):
         tw, ids = self._route(x, md)

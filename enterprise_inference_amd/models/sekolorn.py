@@ -202,6 +202,8 @@ class SekolornForCausalLM(nn.Module):
             if k == "router":
                 return pre + "mlp.router", None
             if k in ("shared.up", "shared.down"):
+                if self.layers[i].mlp.merged_shared:       # stored as expert E
+                    return pre + "mlp.w_" + k[7:], self.layers[i].mlp.E
                 return pre + "mlp." + k + ".weight", None
         return None, None
 

@@ -335,14 +335,19 @@ UNGATED_SMALL_EXPERT = int(os.environ.get("EIA_UNGATED_SMALL_EXPERT", str(2 * 10
 
 def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: int,
                   keep_groups: int, route_scale: float,
-                  row_len: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                  row_len: Optional[torch.Tensor] = None,
+                  always_on: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """Group-limited sigmoid routing (moe.hip route_grouped_kernel): fp32 logits x W_r^T,
     scores = sigmoid; experts form ``num_groups`` equal groups of neighbours, a group scores the
     sum of its two largest scores, only the ``keep_groups`` best groups are eligible, the ``k``
     largest eligible scores win and weigh score * route_scale (not renormalised; ties to the
-    lower index).  -> (weights fp32 [T, k], expert ids int32 [T, k])."""
+    lower index).  -> (weights fp32 [T, k], expert ids int32 [T, k]).
+    ``always_on``: one more column per token naming expert E with weight 1 -- an always-on
+    (shared) expert whose weights are stored behind the E routed ones, so that it rides in the
+    same grouped launches."""
     T, H = x.shape
     E = router_w.shape[0]
+    ko = k + (1 if always_on else 0)
     if not use_hip(x):
         s = torch.sigmoid(x.float() @ router_w.float().t())
         per = E // num_groups
@@ -354,14 +359,19 @@ def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: i
         masked = torch.where(ok[:, :, None].expand(T, num_groups, per).reshape(T, E), s,
                              torch.full_like(s, -1.0))
         order = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :k]
-        return s.gather(1, order) * route_scale, order.to(torch.int32)
+        w, ids = s.gather(1, order) * route_scale, order.to(torch.int32)
+        if always_on:
+            w = torch.cat([w, torch.ones(T, 1)], 1)
+            ids = torch.cat([ids, torch.full((T, 1), E, dtype=torch.int32)], 1)
+        return w, ids
     require(x.stride(1) == 1 and router_w.is_contiguous() and router_w.dtype == x.dtype and
             x.dtype in (torch.bfloat16, torch.float32), "route_grouped: layout")
-    w = torch.empty(T, k, dtype=torch.float32, device=x.device)
-    ids = torch.empty(T, k, dtype=torch.int32, device=x.device)
+    w = torch.empty(T, ko, dtype=torch.float32, device=x.device)
+    ids = torch.empty(T, ko, dtype=torch.int32, device=x.device)
     check(lib().eia_moe_route_grouped(ptr(x), x.stride(0), ptr(router_w), H, T, E, k, num_groups,
                                       keep_groups, float(route_scale), ptr(w), ptr(ids),
-                                      ptr(row_len), 1 if x.dtype == torch.bfloat16 else 0,
+                                      ptr(row_len), 1 if always_on else 0,
+                                      1 if x.dtype == torch.bfloat16 else 0,
                                       stream(x)), "moe_route_grouped")
     return w, ids
 
