@@ -258,3 +258,73 @@ EIA_API int eia_ln_f32in(const float* x, long ldx, const void* w, void* out, lon
                        ldx, (const float*)w, nullptr, (float*)out, ldo, eps, W);
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// RMS norm in groups with an fp32 residual stream.  A row of width W is NG equal consecutive
+// parts; each part is divided by its own sqrt(mean(part^2) + eps) and the row is multiplied by a
+// weight.  One launch does, per row,
+//   x += gnorm(y) * w_post          (y != nullptr: a sublayer's output joins the stream)
+//   x += add                        (add != nullptr: fp32 rows added before the next norm)
+//   h  = gnorm(x) * w_next          (h != nullptr: the next sublayer's input, activation type)
+// so a sublayer boundary (output norm, residual add, next input norm) is one pass over the row.
+// A wave owns whole groups and walks them with the same lane-to-column map in both phases, so a
+// lane re-reads only what it wrote and the row needs no barrier.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gnorm_kernel(const T* __restrict__ y, long ldy, const T* __restrict__ w_post,
+             float* __restrict__ x, const float* __restrict__ add, const T* __restrict__ w_next,
+             T* __restrict__ h, long ldh, float eps, int W, int NG) {
+  const long row = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int gs = W / NG;
+  float* xr = x + row * (long)W;
+  for (int g = wave; g < NG; g += nw) {
+    const int c0 = g * gs;
+    if (y) {
+      const T* yr = y + row * ldy + c0;
+      float ss = 0.f;
+      for (int c = lane; c < gs; c += 64) {
+        const float v = ld_f32<T>(yr, c);
+        ss += v * v;
+      }
+      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+      for (int c = lane; c < gs; c += 64)
+        xr[c0 + c] += ld_f32<T>(yr, c) * inv * ld_f32<T>(w_post, c0 + c);
+    }
+    if (add) {
+      const float* ar = add + row * (long)W + c0;
+      for (int c = lane; c < gs; c += 64) xr[c0 + c] += ar[c];
+    }
+    if (h) {
+      float ss = 0.f;
+      for (int c = lane; c < gs; c += 64) {
+        const float v = xr[c0 + c];
+        ss += v * v;
+      }
+      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+      T* hr = h + row * ldh + c0;
+      for (int c = lane; c < gs; c += 64)
+        st_f32<T>(hr, c, xr[c0 + c] * inv * ld_f32<T>(w_next, c0 + c));
+    }
+  }
+}
+
+// x fp32 [rows, W] contiguous, updated in place when y or add is given; y, w_post, w_next, h are
+// bf16 when is_bf16 else fp32.
+EIA_API int eia_gnorm(const void* y, long ldy, const void* w_post, float* x, const float* add,
+                      const void* w_next, void* h, long ldh, float eps, int rows, int W, int NG,
+                      int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1 || NG < 1 || W % NG || !x || (y && !w_post) || (h && !w_next))
+    return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  const int threads = NG >= 4 ? 256 : 64 * NG;
+  if (is_bf16)
+    hipLaunchKernelGGL((gnorm_kernel<bf16_t>), dim3(rows), dim3(threads), 0, st,
+                       (const bf16_t*)y, ldy, (const bf16_t*)w_post, x, add,
+                       (const bf16_t*)w_next, (bf16_t*)h, ldh, eps, W, NG);
+  else
+    hipLaunchKernelGGL((gnorm_kernel<float>), dim3(rows), dim3(threads), 0, st, (const float*)y,
+                       ldy, (const float*)w_post, x, add, (const float*)w_next, (float*)h, ldh,
+                       eps, W, NG);
+  EIA_LAUNCH_CHECK();
+}

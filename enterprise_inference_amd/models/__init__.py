@@ -18,6 +18,7 @@ _REGISTRY: Dict[str, str] = {
     "Llama4ForCausalLM": "mixtral:Llama4ForCausalLM",
     "OPTForCausalLM": "opt:OPTForCausalLM",
     "Sekolorn": "sekolorn:SekolornForCausalLM",
+    "Vedadra": "vedadra:VedadraForCausalLM",
     "BertModel": "bert:BertEmbeddingModel",
     "XLMRobertaModel": "bert:BertEmbeddingModel",
     "XLMRobertaForSequenceClassification": "bert:CrossEncoderModel",

@@ -9,6 +9,12 @@ returns the mixer output in the activation dtype.
   read another layer's rows).  Runs in the absorbed form (ops/latent_attention.py).
 * ``WKVMixer`` -- token-shift mixing and a per-head matrix-state recurrence with data-dependent
   per-channel decay on per-sequence state slots (ops/wkv.py).
+* ``TalkingWindowAttentionMixer`` -- sliding-window softmax attention without rotation: RMS-normed
+  queries and keys, the un-normed keys as values, a per-head temperature, a linear distance
+  penalty, mixing of the heads' scores before the softmax and a sigmoid output gate.
+* ``DifferentialAttentionMixer`` -- two softmax maps per head over the same values, combined as
+  ``a1 - lambda * a2`` and RMS-normed per head; sliding window plus always-visible first tokens.
+  Both run on token-major paged K / V rows (``PagedKVRows``, ops/window_attention.py).
 """
 
 from __future__ import annotations
@@ -18,6 +24,7 @@ import torch.nn as nn
 
 from ..ops import gemm
 from ..ops import latent_attention as lat_ops
+from ..ops import window_attention as win_ops
 from ..ops import wkv as wkv_ops
 from ..ops.attention import AttentionMetadata
 from ..parallel import state as pstate
@@ -157,3 +164,151 @@ class WKVMixer(nn.Module):
                              md.decode_seq_lens if md.seq_cu is None else None, self.eps,
                              self.heads)
         return gemm.linear(y, self.o)
+
+
+class PagedKVRows:
+    """Paged cache of one attention layer in token-major rows: keys [blocks, block, G*P*D]
+    (normed when written) and values [blocks, block, G*Dv], both in the activation dtype."""
+
+    __slots__ = ("k", "v")
+
+    def __init__(self, k: torch.Tensor, v: torch.Tensor):
+        self.k, self.v = k, v
+
+    @classmethod
+    def allocate(cls, num_blocks: int, block_size: int, k_width: int, v_width: int, dtype, device):
+        # zero filled: never-written rows stay finite under a zero softmax weight
+        return cls(torch.zeros(num_blocks, block_size, k_width, dtype=dtype, device=device),
+                   torch.zeros(num_blocks, block_size, v_width, dtype=dtype, device=device))
+
+
+def _pad64(n: int) -> int:
+    # fused projections are padded with zero rows to a multiple of 64: decode-sized batches then
+    # run the weight-streaming GEMM, whose row tiles need it; the pad columns are never read
+    return -(-n // 64) * 64
+
+
+class _WindowMixerBase(nn.Module):
+    """Shared parts of the mixers over ``PagedKVRows``: one fused input projection whose named
+    slices load separately, per-map RMS norm of queries and keys at cache-write time, the
+    attention launch and the output projection."""
+
+    maps = 1
+
+    def _setup(self, width, heads, kv_heads, dim, vdim, scale, window, keep, eps, parts, bias,
+               dtype, device):
+        if pstate.tp_size() != 1:
+            raise NotImplementedError("window attention mixers run on one rank (no head sharding yet)")
+        if heads % kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+        self.width, self.heads, self.kv_heads, self.dim, self.vdim = width, heads, kv_heads, dim, vdim
+        self.scale, self.window, self.keep, self.eps = float(scale), int(window), int(keep), float(eps)
+        self.offsets, n = {}, 0
+        for name, rows in parts:
+            self.offsets[name] = (n, rows)
+            n += rows
+        self.proj = _param((_pad64(n), width), dtype, device)
+        self.proj.data[n:].zero_()
+        self.proj.weight_loader = self._load_part
+        self.proj_bias = None
+        if bias:
+            self.proj_bias = _param((_pad64(n),), dtype, device)
+            self.proj_bias.data.zero_()
+            self.proj_bias.weight_loader = self._load_part
+        self.q_norm = _plain((dim,), dtype, device)
+        self.k_norm = _plain((dim,), dtype, device)
+        self.o = _plain((width, heads * vdim), dtype, device)
+        M = heads * self.maps
+        # fp32 constants of the attention launch, refreshed IN PLACE after a weight load
+        # (captured decode graphs hold their addresses)
+        self.mult = torch.full((M,), self.scale, dtype=torch.float32, device=device)
+        self.spec = win_ops.WindowSpec(heads, kv_heads, self.maps, dim, vdim, self.window,
+                                       self.keep, self.mult, eps=self.eps)
+        self.qblock = win_ops.query_block(self.spec, dtype if torch.device(device).type == "cuda"
+                                          else torch.float32)
+
+    def _load_part(self, param, loaded, shard_id=None):
+        off, rows = self.offsets[shard_id]
+        if loaded.shape[0] != rows or param.data[off:off + rows].shape != loaded.shape:
+            raise ValueError(f"{type(self).__name__} {shard_id}: shape {tuple(loaded.shape)}")
+        param.data[off:off + rows].copy_(loaded)
+
+    def cache_widths(self):
+        """(key row width, value row width) of this layer's PagedKVRows."""
+        return self.kv_heads * self.maps * self.dim, self.kv_heads * self.vdim
+
+    def refresh(self) -> None:
+        pass
+
+    def _attend(self, xb, md, cache: PagedKVRows, v_part: str, gate_part=None):
+        fused = gemm.linear(xb, self.proj, self.proj_bias)
+        P = self.maps
+        q = win_ops.qk_norm_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
+                                  self.offsets[v_part][0], self.heads * P, self.kv_heads * P,
+                                  self.dim, self.kv_heads * self.vdim, self.q_norm, self.k_norm,
+                                  cache.k, cache.v, md.slot_mapping, self.eps)
+        gate = None
+        if gate_part is not None:
+            g0, gn = self.offsets[gate_part]
+            gate = fused[:, g0:g0 + gn]
+        return win_ops.window_attention(q, cache.k, cache.v, md, self.spec, gate)
+
+
+class TalkingWindowAttentionMixer(_WindowMixerBase):
+    """score_h(i, j) = sum_g talk[h, g] ((q_g . k_j) scale temp_g - slope_g (i - j)) over the
+    window 0 <= i - j < window, slope_g = 2^(-slope_bits (g + 1) / H); values are the keys as
+    projected (before their norm); the heads are gated by sigmoid(W_g x) before W_o.  q, k and
+    the output projection carry biases."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 window: int, eps: float, dtype, device, slope_bits: float = 8.0):
+        super().__init__()
+        if vdim != dim:
+            raise ValueError("values are the projected keys: vdim must equal dim")
+        self._setup(width, heads, kv_heads, dim, vdim, scale, window, 0, eps,
+                    [("q", heads * dim), ("k", kv_heads * dim), ("g", heads * vdim)], True,
+                    dtype, device)
+        self.temp = _plain((heads,), dtype, device)
+        self.talk = _plain((heads, heads), dtype, device)
+        self.o_bias = _plain((width,), dtype, device)
+        h = torch.arange(1, heads + 1, dtype=torch.float64)
+        self.spec.slope = torch.pow(2.0, -float(slope_bits) * h / heads).to(torch.float32).to(device)
+        self.spec.talk = torch.zeros(heads, heads, dtype=torch.float32, device=device)
+
+    def refresh(self) -> None:
+        self.mult.copy_(self.temp.float() * self.scale)
+        self.spec.talk.copy_(self.talk.float())
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
+        return gemm.linear(self._attend(xb, md, cache, "k", "g"), self.o, self.o_bias)
+
+
+class DifferentialAttentionMixer(_WindowMixerBase):
+    """Each head has two query / key maps (rows laid out head by head as [map 1 | map 2]) that
+    attend the same values; lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff is one number for
+    the layer; out_h = rms(a1_h - lambda a2_h) (1 - diff).  Position i sees j <= i with
+    i - j < window or j < keep."""
+
+    maps = 2
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 window: int, keep: int, diff: float, eps: float, dtype, device):
+        super().__init__()
+        self._setup(width, heads, kv_heads, dim, vdim, scale, window, keep, eps,
+                    [("q", heads * 2 * dim), ("k", kv_heads * 2 * dim), ("v", kv_heads * vdim)],
+                    False, dtype, device)
+        self.diff = float(diff)
+        self.lq1, self.lk1 = _plain((dim,), dtype, device), _plain((dim,), dtype, device)
+        self.lq2, self.lk2 = _plain((dim,), dtype, device), _plain((dim,), dtype, device)
+        self.spec.epilogue = 1
+        self.spec.post = 1.0 - self.diff
+        self.spec.lam = self.diff
+
+    def refresh(self) -> None:
+        # a launch constant, baked into captured graphs: refresh before capture
+        a = torch.exp((self.lq1.float() * self.lk1.float()).sum())
+        b = torch.exp((self.lq2.float() * self.lk2.float()).sum())
+        self.spec.lam = float(a - b + self.diff)
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
+        return gemm.linear(self._attend(xb, md, cache, "v"), self.o)

@@ -100,3 +100,51 @@ def layer_norm_f32(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.T
     check(lib().eia_ln_f32in(ptr(x), x.stride(0), ptr(weight), ptr(out), W, float(eps), T, W,
                              1 if bf else 0, stream(x)), "ln_f32in")
     return out
+
+
+def _group_rms(v: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    p = v.reshape(*v.shape[:-1], groups, v.shape[-1] // groups)
+    return (p / torch.sqrt((p * p).mean(-1, keepdim=True) + eps)).reshape(v.shape)
+
+
+def group_norm_step(x: torch.Tensor, groups: int, eps: float, y: Optional[torch.Tensor] = None,
+                    w_post: Optional[torch.Tensor] = None, add: Optional[torch.Tensor] = None,
+                    w_next: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One sublayer boundary of a model whose norms are RMS norms in ``groups`` equal consecutive
+    parts (each part divided by its own root mean square, the row times a weight) around an fp32
+    residual stream x [T, W], in one pass over the row:
+
+        x += gnorm(y) * w_post      (y given: a sublayer's output joins the stream, in place)
+        x += add                    (add given: fp32 rows, in place)
+        h  = gnorm(x) * w_next      (w_next given: returned in the weights' dtype)
+
+    All arithmetic is fp32; y and the weights are in the activation dtype."""
+    T, W = x.shape
+    require(W % groups == 0, "group_norm_step: width not divisible by the group count")
+    if not use_hip(x):
+        if y is not None:
+            x += _group_rms(y.float(), groups, eps) * w_post.float()
+        if add is not None:
+            x += add
+        if w_next is None:
+            return None
+        return (_group_rms(x, groups, eps) * w_next.float()).to(w_next.dtype)
+    ref_w = w_next if w_next is not None else w_post
+    require(x.dtype == torch.float32 and x.is_contiguous(), "group_norm_step: fp32 stream")
+    require(ref_w is not None and ref_w.dtype in (torch.bfloat16, torch.float32),
+            "group_norm_step: bf16 or fp32 weights")
+    bf = ref_w.dtype == torch.bfloat16
+    if y is not None:
+        require(y.shape == x.shape and y.stride(-1) == 1 and y.dtype == ref_w.dtype and
+                w_post.dtype == ref_w.dtype and w_post.numel() == W, "group_norm_step: y layout")
+    if add is not None:
+        require(add.dtype == torch.float32 and add.is_contiguous() and add.shape == x.shape,
+                "group_norm_step: add layout")
+    h = None
+    if w_next is not None:
+        require(w_next.numel() == W, "group_norm_step: weight size")
+        h = torch.empty(T, W, dtype=w_next.dtype, device=x.device)
+    check(lib().eia_gnorm(ptr(y), y.stride(0) if y is not None else 0, ptr(w_post), ptr(x),
+                          ptr(add), ptr(w_next), ptr(h), W, float(eps), T, W, groups,
+                          1 if bf else 0, stream(x)), "gnorm")
+    return h

@@ -1,0 +1,189 @@
+"""Windowed multi-map attention ops -> csrc/kernels/window_attention.hip.
+
+The paged cache of a layer holds two token-major row tensors, keys ``[blocks, block, G*P*D]``
+(RMS-normed at write time) and values ``[blocks, block, G*Dv]``.  A query row carries
+``M = H*P`` score maps (P = 1: ordinary heads; P = 2: the two maps of a differential head);
+map ``h*P + c`` reads key map ``(h // (H//G))*P + c`` and value head ``h // (H//G)``.  Per map
+the score of (query position i, key j) is ``(q.k) * mult[m] - slope[m]*(i-j)``, optionally mixed
+across maps by a matrix (``talk``), masked to ``j <= i and (i-j < window or j < keep)`` and
+soft-maxed.  ``spec.epilogue`` 0 multiplies the heads by ``sigmoid(gate)``; 1 combines a head's
+two maps as ``a1 - lam*a2``, divides by the root mean square over the head and scales.
+
+A step's rows are [decode rows (1 per sequence) | prefill chunks]; both parts read the cache
+after ``qk_norm_cache`` wrote this step's rows, so chunked prompts need no special path.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import List, Optional
+
+import torch
+
+from ._dispatch import check, lib, ptr, require, stream, use_hip
+
+SCALAR_QB = 4            # queries per prefill work item of the scalar-FMA kernel
+
+
+@dataclasses.dataclass
+class WindowSpec:
+    """Constants of one attention layer (device tensors are fp32)."""
+    heads: int
+    kv_heads: int
+    maps: int                       # P: score maps per head
+    dim: int
+    vdim: int
+    window: int                     # 0: no window (every earlier key)
+    keep: int                       # first tokens that stay visible
+    mult: torch.Tensor              # [H*P]
+    slope: Optional[torch.Tensor] = None    # [H*P]
+    talk: Optional[torch.Tensor] = None     # [H*P, H*P]
+    epilogue: int = 0
+    lam: float = 0.0
+    eps: float = 0.0
+    post: float = 1.0
+
+
+def build_work(q_lens: List[int], qblock: int) -> List[int]:
+    """[seq, first query] pairs; a windowed row's work does not grow with its position, so the
+    order is the batch's own."""
+    out: List[int] = []
+    for s, n in enumerate(q_lens):
+        for q0 in range(0, n, qblock):
+            out += [s, q0]
+    return out
+
+
+def query_block(spec: WindowSpec, dtype: torch.dtype) -> int:
+    return SCALAR_QB
+
+
+def _rms(v: torch.Tensor, eps: float) -> torch.Tensor:
+    return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+
+
+def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: int, mk: int,
+                  dim: int, v_width: int, q_w: torch.Tensor, k_w: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                  eps: float) -> torch.Tensor:
+    """One pass over fused projection rows [T, *]: the ``mq`` query maps at ``q_off`` are
+    RMS-normed (weight ``q_w`` [dim]) and returned [T, mq*dim]; the ``mk`` key maps at ``k_off``
+    are RMS-normed (``k_w``) into the token's key row and the ``v_width`` value columns at
+    ``v_off`` (which may be the un-normed key columns) are copied into its value row.  Rows with
+    a slot < 0 write no cache."""
+    T = fused.shape[0]
+    if not use_hip(fused):
+        f = fused.float()
+        q = _rms(f[:, q_off:q_off + mq * dim].reshape(T, mq, dim), eps) * q_w.float()
+        k = _rms(f[:, k_off:k_off + mk * dim].reshape(T, mk, dim), eps) * k_w.float()
+        sm = slot_mapping[:T].long()
+        ok = sm >= 0
+        k_cache.view(-1, k_cache.shape[-1])[sm[ok]] = k.reshape(T, -1)[ok].to(k_cache.dtype)
+        v_cache.view(-1, v_cache.shape[-1])[sm[ok]] = fused[:, v_off:v_off + v_width][ok].to(
+            v_cache.dtype)
+        return q.reshape(T, mq * dim).to(fused.dtype)
+    bf = fused.dtype == torch.bfloat16
+    require(bf or fused.dtype == torch.float32, "qk_norm_cache: bf16 or fp32")
+    require(fused.stride(1) == 1 and max(q_off + mq * dim, k_off + mk * dim, v_off + v_width)
+            <= fused.shape[1], "qk_norm_cache: fused row layout")
+    require(k_cache.dtype == fused.dtype and v_cache.dtype == fused.dtype and
+            k_cache.is_contiguous() and v_cache.is_contiguous() and
+            k_cache.shape[-1] == mk * dim and v_cache.shape[-1] == v_width,
+            "qk_norm_cache: cache layout")
+    require(q_w.dtype == fused.dtype and k_w.dtype == fused.dtype and q_w.numel() == dim and
+            k_w.numel() == dim, "qk_norm_cache: norm weights")
+    require(slot_mapping.dtype == torch.int32 and slot_mapping.numel() >= T, "int32 slots")
+    q = torch.empty(T, mq * dim, dtype=fused.dtype, device=fused.device)
+    check(lib().eia_qk_norm_cache(ptr(fused), fused.stride(0), q_off, k_off, v_off, mq, mk, dim,
+                                  v_width, ptr(q_w), ptr(k_w), ptr(q), q.stride(0), ptr(k_cache),
+                                  ptr(v_cache), ptr(slot_mapping), float(eps), T, 1 if bf else 0,
+                                  stream(fused)), "qk_norm_cache")
+    return q
+
+
+def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpec, seq_of_row):
+    """Plain per-row attention over the paged rows (CPU path)."""
+    H, G, P, D, Dv = spec.heads, spec.kv_heads, spec.maps, spec.dim, spec.vdim
+    rep = H // G
+    bs = k_cache.shape[1]
+    kf = k_cache.view(-1, G, P, D).float()
+    vf = v_cache.view(-1, G, Dv).float()
+    out = torch.zeros(q.shape[0], H * Dv, dtype=torch.float32)
+    for row, s in enumerate(seq_of_row):
+        i = int(positions[row])
+        lo = max(0, i - spec.window + 1) if spec.window > 0 else 0
+        js = torch.tensor(list(range(min(spec.keep, lo))) + list(range(lo, i + 1)))
+        slots = block_table[s].long()[js // bs] * bs + js % bs
+        keys = kf[slots].repeat_interleave(rep, 1).reshape(len(js), H * P, D)      # [n, M, D]
+        vals = vf[slots].repeat_interleave(rep, 1)                                 # [n, H, Dv]
+        sc = torch.einsum("md,nmd->mn", q[row].float().view(H * P, D), keys) * spec.mult[:, None]
+        if spec.slope is not None:
+            sc = sc - spec.slope[:, None] * (i - js).float()[None, :]
+        if spec.talk is not None:
+            sc = spec.talk @ sc
+        w = torch.softmax(sc, -1).view(H, P, len(js))
+        a = torch.einsum("hpn,nhd->hpd", w, vals)
+        if spec.epilogue == 0:
+            o = a[:, 0].reshape(H * Dv)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[row].float())
+        else:
+            o = a[:, 0] - spec.lam * a[:, 1]
+            o = (_rms(o, spec.eps) * spec.post).reshape(H * Dv)
+        out[row] = o
+    return out
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, md,
+                     spec: WindowSpec, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """q [T, H*P*D] (normed; contiguous last dim), gate [T, H*Dv] before the sigmoid or None ->
+    [T, H*Dv] in q's dtype.  ``md`` is the step's AttentionMetadata."""
+    T = q.shape[0]
+    H, P, D, Dv = spec.heads, spec.maps, spec.dim, spec.vdim
+    nd = md.num_decode
+    out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    if not use_hip(q, k_cache):
+        if nd:
+            out[:nd] = _ref_rows(q[:nd], k_cache, v_cache, md.decode_block_tables,
+                                 md.positions[:nd], None if gate is None else gate[:nd], spec,
+                                 list(range(nd))).to(out.dtype)
+        if md.num_prefill_tokens:
+            cu = md.prefill_cu_q.tolist()
+            seqs = [s for s in range(len(cu) - 1) for _ in range(cu[s + 1] - cu[s])]
+            out[nd:] = _ref_rows(q[nd:], k_cache, v_cache, md.prefill_block_tables,
+                                 md.positions[nd:], None if gate is None else gate[nd:], spec,
+                                 seqs).to(out.dtype)
+        return out
+    bf = q.dtype == torch.bfloat16
+    require(bf or q.dtype == torch.float32, "window_attention: bf16 or fp32")
+    require(q.stride(1) == 1 and q.shape[1] == H * P * D and k_cache.dtype == q.dtype and
+            v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
+            k_cache.shape[-1] == spec.kv_heads * P * D and v_cache.shape[-1] == spec.kv_heads * Dv,
+            "window_attention: layout")
+    require(gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and
+                             gate.shape[1] >= H * Dv), "window_attention: gate layout")
+    require(md.positions.dtype == torch.int32, "positions int32")
+    for t in (spec.mult, spec.slope, spec.talk):
+        require(t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous()),
+                "window_attention: fp32 device constants")
+    bs = k_cache.shape[1]
+
+    def launch(lo, n_items, bt, lens, cu, work, qb):
+        require(bt.dtype == torch.int32 and bt.stride(1) == 1, "block tables int32")
+        qa, o = q[lo:], out[lo:]
+        g = None if gate is None else gate[lo:]
+        check(lib().eia_window_attn(
+            ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
+            ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
+            ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0, ptr(o),
+            o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep, qb,
+            spec.epilogue, float(spec.lam), float(spec.eps), float(spec.post), 1 if bf else 0,
+            stream(q)), "window_attn")
+
+    if nd:
+        launch(0, nd, md.decode_block_tables, md.decode_seq_lens, None, None, 1)
+    if md.num_prefill_tokens:
+        qb = query_block(spec, q.dtype)
+        work, n_work = md.prefill_work_for(qb, build_work)
+        launch(nd, n_work, md.prefill_block_tables, None, md.prefill_cu_q, work, qb)
+    return out
