@@ -1,0 +1,68 @@
+"""Vedadra on the MI355X path (HIP kernels; fp32 and bf16 activations) against the plain oracle
+in tests/oracles: every kernel alone, then the whole model through the engine."""
+
+import pytest
+import torch
+
+import vedadra_cases as K
+import vedadra_common as C
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+IDS = ["fp32", "bf16"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("case", [K.case_group_norm, K.case_qk_norm_cache], ids=lambda f: f.__name__)
+def test_kernel(case, dtype):
+    case("cuda", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [
+    # kind, H, G, D, Dv, window, kept first tokens, tokens, page
+    ("talking", 4, 2, 16, 16, 40, 0, 150, 16),
+    ("talking", 1, 1, 24, 24, 7, 0, 90, 16),
+    ("talking", 8, 2, 64, 64, 130, 0, 300, 64),
+    ("talking", 16, 4, 128, 128, 200, 0, 420, 64),
+    ("differential", 4, 1, 16, 24, 40, 5, 150, 16),
+    ("differential", 2, 2, 10, 6, 3, 0, 80, 16),
+    ("differential", 4, 2, 32, 64, 64, 4, 300, 64),
+    ("differential", 8, 2, 64, 128, 150, 6, 400, 64),
+], ids=lambda s: "-".join(map(str, s)))
+def test_window_needle(shape, dtype):
+    kind, H, G, D, Dv, size, keep, n, bs = shape
+    K.case_window_needle("cuda", dtype, kind, H, G, D, Dv, size, keep, n, bs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("cfg", [C.config_a, C.config_b, C.config_c], ids=lambda f: f.__name__)
+def test_layers(cfg, dtype):
+    K.case_layers("cuda", dtype, cfg)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("cfg", [C.config_a, C.config_b, C.config_c], ids=lambda f: f.__name__)
+def test_schedules(cfg, dtype):
+    K.case_schedules("cuda", dtype, cfg, seed=7)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_long_decode(dtype):
+    K.case_long_decode("cuda", dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_generate_through_engine(dtype):
+    K.case_generate("cuda", dtype, C.config_a, expect_graphs=(dtype == torch.bfloat16))
+
+
+def test_generate_graph_decode_config_c():
+    K.case_generate("cuda", torch.bfloat16, C.config_c, expect_graphs=True)
+
+
+def test_native_library_loaded():
+    from enterprise_inference_amd import _native
+    lib = _native.kernels()
+    assert hasattr(lib, "eia_window_attn") and hasattr(lib, "eia_gnorm")
+    assert any("libeia_kernels" in p for p in _native.loaded_native_libraries())
