@@ -1,9 +1,11 @@
-// Windowed multi-map softmax attention over a paged, token-major K / V cache.
+// Windowed multi-map softmax attention over a paged cache: key rows are token-major
+// [blocks, block, G * P * D]; values are stored transposed inside a page, [blocks, G * Dv, block],
+// so that eight consecutive keys of one value column are one 16-byte load.
 //
 // A query row carries M = H * P score maps (H heads, P maps per head: 1 for ordinary heads, 2 for
 // a differential pair), each D wide and already RMS-normed.  Map m = h * P + c of head h reads
 // key map (h / (H / G)) * P + c of the token's key row ([G * P, D], normed at write time) and
-// value head h / (H / G) of its value row ([G, Dv]).  For the pair (query position i, key j):
+// value head h / (H / G) of its value columns ([G, Dv]).  For the pair (query position i, key j):
 //
 //   raw_m  = (q_m . k) * mult[m] - slope[m] * (i - j)            (slope == nullptr: no distance term)
 //   s_h    = sum_g talk[h, g] * raw_g                             (talk == nullptr: s = raw)
@@ -11,7 +13,8 @@
 //   p      = softmax over the visible keys, per map;  a_m = sum_j p_mj v_j
 //
 // Epilogue 0: out[h] = a_h * sigmoid(gate[h])   (gate == nullptr: out = a; P must be 1)
-// Epilogue 1: o = a_{2h} - lam * a_{2h+1};  out[h] = o / sqrt(mean(o^2) + eps) * post   (P == 2)
+// Epilogue 1: o = a_{2h} - lam * a_{2h+1};  out[h] = o / sqrt(mean(o^2) + eps) * post   (P == 2;
+//             lam is read from device memory, so a captured launch follows a weight reload)
 //
 // Scores, softmax weights, accumulators, norms and gates are fp32 whatever the storage type.
 // Rows are [decode rows (one per sequence) | prefill chunks]; both read the cache after
@@ -23,7 +26,7 @@
 // Cache write.  One workgroup per token of a fused projection row:
 //   q maps  -> RMS norm (weight qw[D]) -> q_out[t, MQ * D]
 //   k maps  -> RMS norm (weight kw[D]) -> key row of the token's slot
-//   values  -> copied as projected     -> value row of the token's slot
+//   values  -> copied as projected     -> value columns of the token's slot (page-transposed)
 // (values may alias the un-normed key columns: v_off == k_off).  Slots < 0 write no cache rows.
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -31,7 +34,7 @@ qk_norm_cache_kernel(const T* __restrict__ fused, long ld, int q_off, int k_off,
                      int MQ, int MK, int D, int VW, const T* __restrict__ qw,
                      const T* __restrict__ kw, T* __restrict__ q_out, long ldq,
                      T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots,
-                     float eps) {
+                     int bs, float eps) {
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const T* row = fused + t * ld;
@@ -54,35 +57,35 @@ qk_norm_cache_kernel(const T* __restrict__ fused, long ld, int q_off, int k_off,
   }
   if (slot >= 0) {
     const T* src = row + v_off;
-    T* dst = vc + slot * (long)VW;
-    for (int c = threadIdx.x; c < VW; c += blockDim.x) dst[c] = src[c];
+    T* dst = vc + (slot / bs) * (long)VW * bs + slot % bs;
+    for (int c = threadIdx.x; c < VW; c += blockDim.x) dst[(long)c * bs] = src[c];
   }
 }
 
 EIA_API int eia_qk_norm_cache(const void* fused, long ld, int q_off, int k_off, int v_off, int MQ,
                               int MK, int D, int VW, const void* qw, const void* kw, void* q_out,
-                              long ldq, void* kc, void* vc, const int* slots, float eps, int T,
-                              int is_bf16, hipStream_t st) {
-  if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || !fused || !q_out || !kc || !vc)
+                              long ldq, void* kc, void* vc, const int* slots, int bs, float eps,
+                              int T, int is_bf16, hipStream_t st) {
+  if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || bs < 1 || !fused || !q_out || !kc || !vc)
     return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
   if (is_bf16)
     hipLaunchKernelGGL((qk_norm_cache_kernel<bf16_t>), dim3(T), dim3(256), 0, st,
                        (const bf16_t*)fused, ld, q_off, k_off, v_off, MQ, MK, D, VW,
                        (const bf16_t*)qw, (const bf16_t*)kw, (bf16_t*)q_out, ldq, (bf16_t*)kc,
-                       (bf16_t*)vc, slots, eps);
+                       (bf16_t*)vc, slots, bs, eps);
   else
     hipLaunchKernelGGL((qk_norm_cache_kernel<float>), dim3(T), dim3(256), 0, st,
                        (const float*)fused, ld, q_off, k_off, v_off, MQ, MK, D, VW,
                        (const float*)qw, (const float*)kw, (float*)q_out, ldq, (float*)kc,
-                       (float*)vc, slots, eps);
+                       (float*)vc, slots, bs, eps);
   EIA_LAUNCH_CHECK();
 }
 
 // ---------------------------------------------------------------------------------------------
 struct WinAttnArgs {
   const void* q; long ldq;          // [rows, M * D]
-  const void* kc; const void* vc;   // [slots, G * P * D], [slots, G * Dv]
+  const void* kc; const void* vc;   // [blocks, bs, G * P * D], [blocks, G * Dv, bs]
   const int* bt; int ldbt;          // block tables [seqs, ldbt]
   const int* positions;             // [rows]
   const int* cu;                    // prefill: first row of each sequence's chunk; decode: null
@@ -94,7 +97,8 @@ struct WinAttnArgs {
   const void* gate; long ldg;       // [rows, H * Dv] before the sigmoid, or null
   void* out; long ldo;              // [rows, H * Dv]
   int H, G, P, D, Dv, bs, window, keep, qb, epilogue;
-  float lam, eps, post;
+  const float* lam;                 // [1], epilogue 1
+  float eps, post;
 };
 
 constexpr int WA_KT = 64;           // keys per tile = lanes of a wave
@@ -117,7 +121,7 @@ window_attn_kernel(const WinAttnArgs a) {
   float* mrun = fin + M * Dv;             // [M]
   float* lrun = mrun + M;                 // [M]
   float* alpha = lrun + M;                // [M]
-  long* kslot = reinterpret_cast<long*>(alpha + M + (M & 1));   // [64], 8-byte aligned
+  long* vbase = reinterpret_cast<long*>(alpha + M + (M & 1));   // [64], 8-byte aligned
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const T* q = (const T*)a.q;
   const T* kc = (const T*)a.kc;
@@ -164,7 +168,7 @@ window_attn_kernel(const WinAttnArgs a) {
       const int j = valid ? (kk < nsink ? kk : lo + kk - nsink) : pos;
       const long slot = (long)bt[j / a.bs] * a.bs + j % a.bs;
       __syncthreads();                                 // qs / mrun ready; last tile's reads over
-      if (wave == 0) kslot[lane] = slot;
+      if (wave == 0) vbase[lane] = (long)bt[j / a.bs] * vrow * a.bs + j % a.bs;
       // (1) raw scores of this lane's key
       for (int m = wave; m < M; m += 4) {
         const int h = m / P, c = m - h * P;
@@ -207,10 +211,10 @@ window_attn_kernel(const WinAttnArgs a) {
         const int idx = tid + i * 256;
         if (idx < M * Dv) {
           const int m = idx / Dv, d = idx - m * Dv;
-          const T* vp = vc + ((m / P) / rep) * Dv + d;
+          const T* vp = vc + (long)(((m / P) / rep) * Dv + d) * a.bs;
           const float* pm = pw + m * WA_KT;
           float s = acc[i] * alpha[m];
-          for (int k = 0; k < nk; ++k) s += pm[k] * ld_f32<T>(vp, kslot[k] * vrow);
+          for (int k = 0; k < nk; ++k) s += pm[k] * ld_f32<T>(vp, vbase[k]);
           acc[i] = s;
         }
       }
@@ -233,17 +237,18 @@ window_attn_kernel(const WinAttnArgs a) {
         if (idx < M * Dv) fin[idx] = acc[i] / lrun[idx / Dv];
       }
       __syncthreads();
+      const float lam = a.lam[0];
       for (int h = wave; h < H; h += 4) {
         const float* a1 = fin + (2 * h) * Dv;
         const float* a2 = a1 + Dv;
         float ss = 0.f;
         for (int d = lane; d < Dv; d += 64) {
-          const float o = a1[d] - a.lam * a2[d];
+          const float o = a1[d] - lam * a2[d];
           ss += o * o;
         }
         const float inv = a.post / sqrtf(wave_sum(ss) / (float)Dv + a.eps);
         for (int d = lane; d < Dv; d += 64)
-          st_f32<T>(out + row * a.ldo, h * Dv + d, (a1[d] - a.lam * a2[d]) * inv);
+          st_f32<T>(out + row * a.ldo, h * Dv + d, (a1[d] - lam * a2[d]) * inv);
       }
     }
   }
@@ -260,13 +265,15 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
                             const int* lens, int n_items, const float* mult, const float* slope,
                             const float* talk, const void* gate, long ldg, void* out, long ldo,
                             int H, int G, int P, int D, int Dv, int bs, int window, int keep,
-                            int qb, int epilogue, float lam, float eps, float post, int is_bf16,
+                            int qb, int epilogue, const float* lam, float eps, float post,
+                            int is_bf16,
                             hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || D < 1 || Dv < 1 || bs < 1 ||
       keep < 0 || qb < 1 || !q || !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
-  if ((epilogue == 1) != (P == 2) || (epilogue == 1 && gate)) return EIA_BAD_SHAPE;
+  if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam)))
+    return EIA_BAD_SHAPE;
   const int M = H * P;
   const size_t lds = wa_lds_bytes(M, D, Dv);
   if (M * Dv > 256 * WA_ACC || lds > 64 * 1024) return EIA_UNSUPPORTED;
@@ -277,5 +284,323 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
     hipLaunchKernelGGL((window_attn_kernel<bf16_t>), dim3(n_items), dim3(256), lds, st, a);
   else
     hipLaunchKernelGGL((window_attn_kernel<float>), dim3(n_items), dim3(256), lds, st, a);
+  EIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------
+// MFMA form (bf16): v_mfma_f32_16x16x32_bf16, operands straight from the cache into registers.
+//
+// A workgroup of NWV waves owns a tile of 16 queries of one sequence and NWV * HW heads; a wave
+// owns HW heads (HW * P maps) and walks the visible keys in absolute 32-key blocks (a block
+// never straddles a page: block size % 32 == 0), first the blocks of the kept first tokens that
+// lie before the window, then the window's.  Per block and map it forms S^T (keys x queries)
+// as two 16-key tiles whose rows are ordered so that the accumulator registers of a lane --
+// query lane % 16, keys 8 (lane / 16) + e -- are the B operand of the second product,
+// O^T (value columns x queries) += V^T P^T, with V^T read as eight consecutive keys of a value
+// column (the page-transposed value layout).  Nothing passes through LDS except, with head
+// mixing, the raw scores: every wave writes its maps' tiles, one barrier, every wave reads all
+// maps and mixes the rows of its own heads (buffers alternate between blocks).
+// Softmax weights stay fp32: P enters the second product as a bf16 high part plus a bf16
+// remainder, and the normaliser sums the fp32 weights.
+template <int HW, int P, bool TALK, int ND, int NDV>
+__global__ void __launch_bounds__(256)
+window_attn_mfma_kernel(const WinAttnArgs a) {
+  constexpr int MW = HW * P;
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int H = a.H, D = a.D, Dv = a.Dv, M = H * P, rep = H / a.G, bs = a.bs;
+  const int nd = (D + 31) >> 5, ndv = Dv >> 4;
+  const bf16_t* q = (const bf16_t*)a.q;
+  const bf16_t* kc = (const bf16_t*)a.kc;
+  const bf16_t* vc = (const bf16_t*)a.vc;
+  const long krow = (long)a.G * P * D, vpage = (long)a.G * Dv * bs;
+
+  int seq, row0, nq;
+  if (a.cu) {
+    seq = a.work[2 * blockIdx.x];
+    const int q0 = a.work[2 * blockIdx.x + 1];
+    row0 = a.cu[seq] + q0;
+    nq = min(16, a.cu[seq + 1] - a.cu[seq] - q0);
+  } else {
+    seq = blockIdx.x;
+    row0 = seq;
+    nq = (a.lens && a.lens[seq] <= 0) ? 0 : 1;
+  }
+  const int h0 = (blockIdx.y * (blockDim.x >> 6) + wave) * HW;      // this wave's first head
+  const bool wave_on = h0 < H;                                      // (H % HW == 0)
+  const int* bt = a.bt + (long)seq * a.ldbt;
+  bf16_t* out = (bf16_t*)a.out;
+  if (nq == 0) {                                                    // padding row: zeros
+    if (wave_on)
+      for (int i = lane; i < HW * Dv; i += 64) out[(long)row0 * a.ldo + h0 * Dv + i] = f2bf(0.f);
+    return;
+  }
+  const bool row_ok = c < nq;
+  const long row = row0 + (row_ok ? c : 0);
+  const int qpos = a.positions[row];
+  const int pos_first = a.positions[row0], pos_last = a.positions[row0 + nq - 1];
+  const int lo_min = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
+  const int wb0 = lo_min >> 5, wb1 = pos_last >> 5;                 // window blocks wb0 .. wb1
+  const int nsink = min((min(a.keep, lo_min) + 31) >> 5, wb0);      // kept-token blocks before wb0
+  const int nblocks = nsink + wb1 - wb0 + 1;
+
+  // Q^T operands of this wave's maps: column = query c, rows = d 32 s + 8 g .. + 8
+  bf16x8 qf[MW][ND];
+#pragma unroll
+  for (int m = 0; m < MW; ++m)
+#pragma unroll
+    for (int s = 0; s < ND; ++s) {
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      const int d = 32 * s + 8 * g;
+      if (wave_on && s < nd && d < D)
+        v = *reinterpret_cast<const bf16x8*>(q + row * a.ldq + (h0 * P + m) * D + d);
+      qf[m][s] = v;
+    }
+  float mult[MW], slope[MW];
+#pragma unroll
+  for (int m = 0; m < MW; ++m) {
+    mult[m] = wave_on ? a.mult[h0 * P + m] : 0.f;
+    slope[m] = (wave_on && a.slope) ? a.slope[h0 * P + m] : 0.f;
+  }
+  f32x4 acc[MW][NDV];
+  float mrun[MW], lrun[MW];
+#pragma unroll
+  for (int m = 0; m < MW; ++m) {
+    mrun[m] = -1e30f;
+    lrun[m] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NDV; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int b = 0; b < nblocks; ++b) {
+    const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
+    const int key0 = kb << 5;
+    const long page = bt[key0 / bs];
+    const int off = key0 % bs;
+    // S^T tiles: tile t, row 4 g' + i  <->  key 8 g' + 4 t + i; this lane's A rows are c
+    const int r0 = 8 * (c >> 2) + (c & 3);                          // key of row c in tile 0
+    const bf16_t* k0p = kc + (page * bs + off + r0) * krow;
+    const bf16_t* k1p = k0p + 4 * krow;
+    f32x4 sc[MW][2];
+#pragma unroll
+    for (int m = 0; m < MW; ++m) {
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+      if (wave_on) {
+        const int km = (((h0 + m / P) / rep) * P + m % P) * D;
+#pragma unroll
+        for (int s = 0; s < ND; ++s) {
+          const int d = 32 * s + 8 * g;
+          if (s < nd) {
+            bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb2 = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (d < D) {
+              ka = *reinterpret_cast<const bf16x8*>(k0p + km + d);
+              kb2 = *reinterpret_cast<const bf16x8*>(k1p + km + d);
+            }
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[m][s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2, qf[m][s], s1, 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ka = key0 + 8 * g + i;
+        s0[i] = s0[i] * mult[m] - slope[m] * (float)(qpos - ka);
+        s1[i] = s1[i] * mult[m] - slope[m] * (float)(qpos - ka - 4);
+      }
+      sc[m][0] = s0;
+      sc[m][1] = s1;
+    }
+    if constexpr (TALK) {
+      // raw scores of every map through LDS: [buffer][map][tile][lane] f32x4
+      f32x4* buf = reinterpret_cast<f32x4*>(lds) + (size_t)(b & 1) * M * 128;
+      if (wave_on) {
+#pragma unroll
+        for (int m = 0; m < MW; ++m) {
+          buf[((h0 + m) * 2 + 0) * 64 + lane] = sc[m][0];
+          buf[((h0 + m) * 2 + 1) * 64 + lane] = sc[m][1];
+        }
+      }
+      __syncthreads();
+      if (wave_on) {
+#pragma unroll
+        for (int m = 0; m < MW; ++m) {
+          sc[m][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+          sc[m][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        for (int gm = 0; gm < M; ++gm) {
+          const f32x4 r0v = buf[(gm * 2 + 0) * 64 + lane], r1v = buf[(gm * 2 + 1) * 64 + lane];
+#pragma unroll
+          for (int m = 0; m < MW; ++m) {
+            const float tw = a.talk[(h0 + m) * M + gm];
+            sc[m][0] += tw * r0v;
+            sc[m][1] += tw * r1v;
+          }
+        }
+      }
+    }
+    if (!wave_on) continue;
+    // mask, running max / sum, P^T operands
+    bf16x8 ph[MW], pl[MW];
+    float alpha[MW];
+#pragma unroll
+    for (int m = 0; m < MW; ++m) {
+      float v[8];
+      bool vis[8];
+      float mloc = -1e30f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = key0 + 8 * g + e;
+        vis[e] = row_ok && key <= qpos && (a.window <= 0 || qpos - key < a.window || key < a.keep);
+        v[e] = e < 4 ? sc[m][0][e] : sc[m][1][e - 4];
+        if (vis[e]) mloc = fmaxf(mloc, v[e]);
+      }
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
+      mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
+      const float mnew = fmaxf(mrun[m], mloc);
+      alpha[m] = expf(mrun[m] - mnew);
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = vis[e] ? expf(v[e] - mnew) : 0.f;
+        const bf16_t hi = f2bf(p);
+        ph[m][e] = hi;
+        pl[m][e] = f2bf(p - bf2f(hi));
+        psum += p;
+      }
+      psum += __shfl_xor(psum, 16, 64);
+      psum += __shfl_xor(psum, 32, 64);
+      lrun[m] = lrun[m] * alpha[m] + psum;
+      mrun[m] = mnew;
+    }
+    // O^T += V^T P^T: A rows = value columns 16 t + c, k = keys 8 g .. + 8 of the block
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const bf16_t* vp = vc + page * vpage + ((long)((h0 + hh) / rep) * Dv + c) * bs + off + 8 * g;
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) {
+        if (t < ndv) {
+          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vp + (long)t * 16 * bs);
+#pragma unroll
+          for (int pm = 0; pm < P; ++pm) {
+            const int m = hh * P + pm;
+            f32x4 o = acc[m][t] * alpha[m];
+            o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[m], o, 0, 0, 0);
+            acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[m], o, 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+  if (!wave_on || !row_ok) return;
+  // this lane holds, per map and tile t, value columns 16 t + 4 g + i of query c
+  if (a.epilogue == 0) {
+    const bf16_t* gate = (const bf16_t*)a.gate;
+#pragma unroll
+    for (int m = 0; m < MW; ++m) {
+      const float inv = 1.0f / lrun[m];
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) {
+        if (t < ndv) {
+          const int col = (h0 + m) * Dv + 16 * t + 4 * g;
+          bf16x4 o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float v = acc[m][t][i] * inv;
+            if (gate) v *= 1.0f / (1.0f + expf(-bf2f(gate[row * a.ldg + col + i])));
+            o[i] = f2bf(v);
+          }
+          *reinterpret_cast<bf16x4*>(out + row * a.ldo + col) = o;
+        }
+      }
+    }
+  } else {
+    const float lam = a.lam[0];
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const float i1 = 1.0f / lrun[2 * hh], i2 = lam / lrun[2 * hh + 1];
+      float ss = 0.f;
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) {
+        if (t < ndv) {
+          const f32x4 o = acc[2 * hh][t] * i1 - acc[2 * hh + 1][t] * i2;
+          acc[2 * hh][t] = o;
+          ss += o[0] * o[0] + o[1] * o[1] + o[2] * o[2] + o[3] * o[3];
+        }
+      }
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      const float inv = a.post / sqrtf(ss / (float)Dv + a.eps);
+#pragma unroll
+      for (int t = 0; t < NDV; ++t) {
+        if (t < ndv) {
+          bf16x4 o;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[i] = f2bf(acc[2 * hh][t][i] * inv);
+          *reinterpret_cast<bf16x4*>(out + row * a.ldo + (h0 + hh) * Dv + 16 * t + 4 * g) = o;
+        }
+      }
+    }
+  }
+}
+
+// Heads per wave of the MFMA form for (H, P), 0 when the shape runs the scalar form: with head
+// mixing one workgroup must hold every head (H / HW <= 4 waves); without it the heads are
+// spread over grid.y in workgroups of up to four single-head waves.
+static int wa_mfma_hw(int H, int P, int talk) {
+  if (!talk) return 1;
+  if (P != 1) return 0;
+  if (H <= 4) return 1;
+  if (H <= 8 && H % 2 == 0) return 2;
+  if (H <= 16 && H % 4 == 0) return 4;
+  return 0;
+}
+
+EIA_API int eia_window_attn_mfma_ok(int H, int P, int D, int Dv, int bs, int talk) {
+  return wa_mfma_hw(H, P, talk) > 0 && D % 8 == 0 && D <= 128 && Dv % 16 == 0 && Dv <= 128 &&
+         bs % 32 == 0;
+}
+
+EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const void* vc,
+                                 const int* bt, int ldbt, const int* positions, const int* cu,
+                                 const int* work, const int* lens, int n_items, const float* mult,
+                                 const float* slope, const float* talk, const void* gate, long ldg,
+                                 void* out, long ldo, int H, int G, int P, int D, int Dv, int bs,
+                                 int window, int keep, int epilogue, const float* lam, float eps,
+                                 float post, hipStream_t st) {
+  if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || bs < 1 || keep < 0 || !q ||
+      !kc || !vc || !bt || !positions || !mult || !out)
+    return EIA_BAD_SHAPE;
+  if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
+  if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam))) return EIA_BAD_SHAPE;
+  if (!eia_window_attn_mfma_ok(H, P, D, Dv, bs, talk != nullptr)) return EIA_UNSUPPORTED;
+  if (ldq % 8 || ldo % 4 || (gate && ldg % 1)) return EIA_BAD_SHAPE;
+  if (n_items == 0) return EIA_OK;
+  WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
+                out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post};
+  const int hw = wa_mfma_hw(H, P, talk != nullptr);
+  const int waves_needed = H / hw;
+  const int nwv = talk ? waves_needed : (waves_needed < 4 ? waves_needed : 4);
+  const int gy = talk ? 1 : (waves_needed + nwv - 1) / nwv;
+  const size_t lds = talk ? (size_t)2 * H * P * 128 * sizeof(f32x4) : 0;
+  const bool big = D > 64 || Dv > 64;
+  dim3 grid(n_items, gy), block(64 * nwv);
+#define WA_LAUNCH(HWV, PV, TK)                                                                  \
+  do {                                                                                          \
+    if (big)                                                                                    \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<HWV, PV, TK, 4, 8>), grid, block, lds, st, a); \
+    else                                                                                        \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<HWV, PV, TK, 2, 4>), grid, block, lds, st, a); \
+  } while (0)
+  if (talk) {
+    if (hw == 1) WA_LAUNCH(1, 1, true);
+    else if (hw == 2) WA_LAUNCH(2, 1, true);
+    else WA_LAUNCH(4, 1, true);
+  } else if (P == 2) {
+    WA_LAUNCH(1, 2, false);
+  } else {
+    WA_LAUNCH(1, 1, false);
+  }
+#undef WA_LAUNCH
   EIA_LAUNCH_CHECK();
 }

@@ -167,8 +167,9 @@ class WKVMixer(nn.Module):
 
 
 class PagedKVRows:
-    """Paged cache of one attention layer in token-major rows: keys [blocks, block, G*P*D]
-    (normed when written) and values [blocks, block, G*Dv], both in the activation dtype."""
+    """Paged cache of one attention layer: token-major key rows [blocks, block, G*P*D] (normed
+    when written) and values transposed inside a page, [blocks, G*Dv, block], both in the
+    activation dtype."""
 
     __slots__ = ("k", "v")
 
@@ -179,7 +180,7 @@ class PagedKVRows:
     def allocate(cls, num_blocks: int, block_size: int, k_width: int, v_width: int, dtype, device):
         # zero filled: never-written rows stay finite under a zero softmax weight
         return cls(torch.zeros(num_blocks, block_size, k_width, dtype=dtype, device=device),
-                   torch.zeros(num_blocks, block_size, v_width, dtype=dtype, device=device))
+                   torch.zeros(num_blocks, v_width, block_size, dtype=dtype, device=device))
 
 
 def _pad64(n: int) -> int:
@@ -224,14 +225,17 @@ class _WindowMixerBase(nn.Module):
         self.mult = torch.full((M,), self.scale, dtype=torch.float32, device=device)
         self.spec = win_ops.WindowSpec(heads, kv_heads, self.maps, dim, vdim, self.window,
                                        self.keep, self.mult, eps=self.eps)
-        self.qblock = win_ops.query_block(self.spec, dtype if torch.device(device).type == "cuda"
-                                          else torch.float32)
+        self._qdtype = dtype if torch.device(device).type == "cuda" else torch.float32
 
     def _load_part(self, param, loaded, shard_id=None):
         off, rows = self.offsets[shard_id]
         if loaded.shape[0] != rows or param.data[off:off + rows].shape != loaded.shape:
             raise ValueError(f"{type(self).__name__} {shard_id}: shape {tuple(loaded.shape)}")
         param.data[off:off + rows].copy_(loaded)
+
+    def query_block(self, block_size: int) -> int:
+        """Queries per prefill work item of this layer's attention kernel."""
+        return win_ops.query_block(self.spec, self._qdtype, block_size)
 
     def cache_widths(self):
         """(key row width, value row width) of this layer's PagedKVRows."""
@@ -302,13 +306,12 @@ class DifferentialAttentionMixer(_WindowMixerBase):
         self.lq2, self.lk2 = _plain((dim,), dtype, device), _plain((dim,), dtype, device)
         self.spec.epilogue = 1
         self.spec.post = 1.0 - self.diff
-        self.spec.lam = self.diff
+        self.spec.lam = torch.full((1,), self.diff, dtype=torch.float32, device=device)
 
     def refresh(self) -> None:
-        # a launch constant, baked into captured graphs: refresh before capture
         a = torch.exp((self.lq1.float() * self.lk1.float()).sum())
         b = torch.exp((self.lq2.float() * self.lk2.float()).sum())
-        self.spec.lam = float(a - b + self.diff)
+        self.spec.lam.copy_((a - b + self.diff).reshape(1))
 
     def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
         return gemm.linear(self._attend(xb, md, cache, "v"), self.o)

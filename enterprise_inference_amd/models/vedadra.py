@@ -142,7 +142,7 @@ class VedadraForCausalLM(nn.Module):
         return out
 
     def prefill_query_block(self, block_size: int) -> int:
-        return self.layers[self.runs[0][0]].mix.qblock if self.runs else 16
+        return self.layers[self.runs[0][0]].mix.query_block(block_size) if self.runs else 16
 
     # ------------------------------------------------------------------ forward
     def forward(self, input_ids: torch.Tensor, md: AttentionMetadata, caches: list,

@@ -1,7 +1,8 @@
 """Windowed multi-map attention ops -> csrc/kernels/window_attention.hip.
 
-The paged cache of a layer holds two token-major row tensors, keys ``[blocks, block, G*P*D]``
-(RMS-normed at write time) and values ``[blocks, block, G*Dv]``.  A query row carries
+The paged cache of a layer holds token-major key rows ``[blocks, block, G*P*D]`` (RMS-normed
+at write time) and values transposed inside a page, ``[blocks, G*Dv, block]`` (eight consecutive
+keys of a value column are one 16-byte load).  A query row carries
 ``M = H*P`` score maps (P = 1: ordinary heads; P = 2: the two maps of a differential head);
 map ``h*P + c`` reads key map ``(h // (H//G))*P + c`` and value head ``h // (H//G)``.  Per map
 the score of (query position i, key j) is ``(q.k) * mult[m] - slope[m]*(i-j)``, optionally mixed
@@ -16,6 +17,7 @@ after ``qk_norm_cache`` wrote this step's rows, so chunked prompts need no speci
 from __future__ import annotations
 
 import dataclasses
+import os
 from typing import List, Optional
 
 import torch
@@ -23,6 +25,8 @@ import torch
 from ._dispatch import check, lib, ptr, require, stream, use_hip
 
 SCALAR_QB = 4            # queries per prefill work item of the scalar-FMA kernel
+MFMA_QB = 16             # ... and of the MFMA kernel (one 16-row tile)
+_MFMA_ENV = os.environ.get("EIA_WINDOW_MFMA", "1") != "0"
 
 
 @dataclasses.dataclass
@@ -39,7 +43,7 @@ class WindowSpec:
     slope: Optional[torch.Tensor] = None    # [H*P]
     talk: Optional[torch.Tensor] = None     # [H*P, H*P]
     epilogue: int = 0
-    lam: float = 0.0
+    lam: Optional[torch.Tensor] = None      # [1], the differential weight (epilogue 1)
     eps: float = 0.0
     post: float = 1.0
 
@@ -54,8 +58,18 @@ def build_work(q_lens: List[int], qblock: int) -> List[int]:
     return out
 
 
-def query_block(spec: WindowSpec, dtype: torch.dtype) -> int:
-    return SCALAR_QB
+def mfma_ok(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> bool:
+    """The MFMA kernel takes bf16 rows with D % 8 == 0, Dv % 16 == 0, both <= 128, pages of a
+    multiple of 32 tokens and, with head mixing, at most 16 heads in 1, 2 or 4 heads per wave;
+    everything else (fp32 models too) runs the scalar-FMA kernel."""
+    if dtype != torch.bfloat16 or not _MFMA_ENV or not torch.cuda.is_available():
+        return False
+    return bool(lib().eia_window_attn_mfma_ok(spec.heads, spec.maps, spec.dim, spec.vdim,
+                                              block_size, 1 if spec.talk is not None else 0))
+
+
+def query_block(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> int:
+    return MFMA_QB if mfma_ok(spec, dtype, block_size) else SCALAR_QB
 
 
 def _rms(v: torch.Tensor, eps: float) -> torch.Tensor:
@@ -79,8 +93,8 @@ def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: i
         sm = slot_mapping[:T].long()
         ok = sm >= 0
         k_cache.view(-1, k_cache.shape[-1])[sm[ok]] = k.reshape(T, -1)[ok].to(k_cache.dtype)
-        v_cache.view(-1, v_cache.shape[-1])[sm[ok]] = fused[:, v_off:v_off + v_width][ok].to(
-            v_cache.dtype)
+        bs = v_cache.shape[2]
+        v_cache[sm[ok] // bs, :, sm[ok] % bs] = fused[:, v_off:v_off + v_width][ok].to(v_cache.dtype)
         return q.reshape(T, mq * dim).to(fused.dtype)
     bf = fused.dtype == torch.bfloat16
     require(bf or fused.dtype == torch.float32, "qk_norm_cache: bf16 or fp32")
@@ -88,7 +102,8 @@ def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: i
             <= fused.shape[1], "qk_norm_cache: fused row layout")
     require(k_cache.dtype == fused.dtype and v_cache.dtype == fused.dtype and
             k_cache.is_contiguous() and v_cache.is_contiguous() and
-            k_cache.shape[-1] == mk * dim and v_cache.shape[-1] == v_width,
+            k_cache.shape[-1] == mk * dim and v_cache.shape[1] == v_width and
+            v_cache.shape[2] == k_cache.shape[1],
             "qk_norm_cache: cache layout")
     require(q_w.dtype == fused.dtype and k_w.dtype == fused.dtype and q_w.numel() == dim and
             k_w.numel() == dim, "qk_norm_cache: norm weights")
@@ -96,7 +111,8 @@ def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: i
     q = torch.empty(T, mq * dim, dtype=fused.dtype, device=fused.device)
     check(lib().eia_qk_norm_cache(ptr(fused), fused.stride(0), q_off, k_off, v_off, mq, mk, dim,
                                   v_width, ptr(q_w), ptr(k_w), ptr(q), q.stride(0), ptr(k_cache),
-                                  ptr(v_cache), ptr(slot_mapping), float(eps), T, 1 if bf else 0,
+                                  ptr(v_cache), ptr(slot_mapping), k_cache.shape[1], float(eps), T,
+                                  1 if bf else 0,
                                   stream(fused)), "qk_norm_cache")
     return q
 
@@ -107,7 +123,7 @@ def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpe
     rep = H // G
     bs = k_cache.shape[1]
     kf = k_cache.view(-1, G, P, D).float()
-    vf = v_cache.view(-1, G, Dv).float()
+    vf = v_cache.permute(0, 2, 1).reshape(-1, G, Dv).float()
     out = torch.zeros(q.shape[0], H * Dv, dtype=torch.float32)
     for row, s in enumerate(seq_of_row):
         i = int(positions[row])
@@ -128,7 +144,7 @@ def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpe
             if gate is not None:
                 o = o * torch.sigmoid(gate[row].float())
         else:
-            o = a[:, 0] - spec.lam * a[:, 1]
+            o = a[:, 0] - float(spec.lam[0]) * a[:, 1]
             o = (_rms(o, spec.eps) * spec.post).reshape(H * Dv)
         out[row] = o
     return out
@@ -158,32 +174,46 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     require(bf or q.dtype == torch.float32, "window_attention: bf16 or fp32")
     require(q.stride(1) == 1 and q.shape[1] == H * P * D and k_cache.dtype == q.dtype and
             v_cache.dtype == q.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
-            k_cache.shape[-1] == spec.kv_heads * P * D and v_cache.shape[-1] == spec.kv_heads * Dv,
+            k_cache.shape[-1] == spec.kv_heads * P * D and v_cache.shape[1] == spec.kv_heads * Dv
+            and v_cache.shape[2] == k_cache.shape[1],
             "window_attention: layout")
     require(gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and
                              gate.shape[1] >= H * Dv), "window_attention: gate layout")
     require(md.positions.dtype == torch.int32, "positions int32")
-    for t in (spec.mult, spec.slope, spec.talk):
+    for t in (spec.mult, spec.slope, spec.talk, spec.lam):
         require(t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous()),
                 "window_attention: fp32 device constants")
     bs = k_cache.shape[1]
+
+    mfma = mfma_ok(spec, q.dtype, bs)
+    if mfma:
+        require(q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0, "window_attention: q alignment")
 
     def launch(lo, n_items, bt, lens, cu, work, qb):
         require(bt.dtype == torch.int32 and bt.stride(1) == 1, "block tables int32")
         qa, o = q[lo:], out[lo:]
         g = None if gate is None else gate[lo:]
+        if mfma:
+            check(lib().eia_window_attn_mfma(
+                ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
+                ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
+                ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0,
+                ptr(o), o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep,
+                spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), stream(q)),
+                "window_attn_mfma")
+            return
         check(lib().eia_window_attn(
             ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
             ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
             ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0, ptr(o),
             o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep, qb,
-            spec.epilogue, float(spec.lam), float(spec.eps), float(spec.post), 1 if bf else 0,
+            spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), 1 if bf else 0,
             stream(q)), "window_attn")
 
     if nd:
         launch(0, nd, md.decode_block_tables, md.decode_seq_lens, None, None, 1)
     if md.num_prefill_tokens:
-        qb = query_block(spec, q.dtype)
+        qb = query_block(spec, q.dtype, bs)
         work, n_work = md.prefill_work_for(qb, build_work)
         launch(nd, n_work, md.prefill_block_tables, None, md.prefill_cu_q, work, qb)
     return out

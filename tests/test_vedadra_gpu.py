@@ -29,6 +29,15 @@ def test_kernel(case, dtype):
     ("differential", 2, 2, 10, 6, 3, 0, 80, 16),
     ("differential", 4, 2, 32, 64, 64, 4, 300, 64),
     ("differential", 8, 2, 64, 128, 150, 6, 400, 64),
+    # bf16: the matrix-core form's variants (1, 2, 4 heads per wave; partial last wave; head sizes
+    # that are not multiples of 32; 32-token pages; kept tokens beyond one 32-key block)
+    ("talking", 3, 1, 96, 96, 72, 0, 260, 64),
+    ("talking", 6, 3, 48, 48, 33, 0, 200, 32),
+    ("talking", 12, 4, 32, 32, 100, 0, 300, 32),
+    ("talking", 2, 2, 128, 128, 31, 0, 130, 32),
+    ("differential", 5, 1, 48, 96, 40, 6, 260, 64),
+    ("differential", 1, 1, 24, 16, 64, 40, 300, 32),
+    ("differential", 3, 3, 128, 112, 90, 33, 350, 64),
 ], ids=lambda s: "-".join(map(str, s)))
 def test_window_needle(shape, dtype):
     kind, H, G, D, Dv, size, keep, n, bs = shape
@@ -48,13 +57,19 @@ def test_schedules(cfg, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_schedules_pages_of_32(dtype):
+    """Pages of 32 tokens: the bf16 run takes the matrix-core attention form end to end."""
+    K.case_schedules("cuda", dtype, C.config_c, seed=3, block_size=32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_long_decode(dtype):
     K.case_long_decode("cuda", dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_generate_through_engine(dtype):
-    K.case_generate("cuda", dtype, C.config_a, expect_graphs=(dtype == torch.bfloat16))
+    K.case_generate("cuda", dtype, C.config_a, expect_graphs=True)
 
 
 def test_generate_graph_decode_config_c():

@@ -86,7 +86,7 @@ def case_qk_norm_cache(device, dtype):
         kw = (1 + 0.3 * torch.randn(D, generator=g)).to(dtype)
         slots = torch.tensor([9, 2, -1, 17, 0, 5, 19], dtype=torch.int32)
         kc = torch.full((nb, bs, mk * D), 7.0, dtype=dtype)
-        vc = torch.full((nb, bs, vw), 7.0, dtype=dtype)
+        vc = torch.full((nb, vw, bs), 7.0, dtype=dtype)
         kd, vd = kc.to(device), vc.to(device)
         q = wa.qk_norm_cache(fused.to(device), q_off, k_off, v_off, mq, mk, D, vw, qw.to(device),
                              kw.to(device), kd, vd, slots.to(device), 1e-5)
@@ -95,7 +95,8 @@ def case_qk_norm_cache(device, dtype):
             for m in range(mq):
                 want = O.rms_div(f[t, q_off + m * D:q_off + (m + 1) * D], 1e-5) * _np(qw)
                 assert np.allclose(_np(q[t, m * D:(m + 1) * D]), want, atol=ktol(dtype), rtol=ktol(dtype))
-        kflat, vflat = _np(kd).reshape(nb * bs, -1), _np(vd).reshape(nb * bs, -1)
+        kflat = _np(kd).reshape(nb * bs, -1)
+        vflat = _np(vd.permute(0, 2, 1)).reshape(nb * bs, -1)
         used = set()
         for t, s in enumerate(slots.tolist()):
             if s < 0:
@@ -166,7 +167,8 @@ def case_window_needle(device, dtype, kind="talking", H=4, G=2, D=16, Dv=16, siz
         spec.slope = torch.pow(2.0, -8.0 * hh / H).float().to(device)
         spec.talk = talk.to(device)
     else:
-        spec.epilogue, spec.lam, spec.eps, spec.post = 1, lam, 1e-5, 1.0 - diff
+        spec.epilogue, spec.eps, spec.post = 1, 1e-5, 1.0 - diff
+        spec.lam = torch.tensor([lam], dtype=torch.float32, device=device)
     for j in sorted(c for c in cand if 0 <= c <= i):
         q = torch.randn(n, H * P, D, generator=g) * 0.5
         k = torch.randn(n, G * P, D, generator=g) * 0.5
@@ -178,9 +180,9 @@ def case_window_needle(device, dtype, kind="talking", H=4, G=2, D=16, Dv=16, siz
         k[j] += 12.0 * u                       # ... meets every key map of token j
         q, k, v, gate = q.to(dtype), k.to(dtype), v.to(dtype), gate.to(dtype)
         kc = torch.zeros(nblk, bs, G * P * D, dtype=dtype)
-        vc = torch.zeros(nblk, bs, G * Dv, dtype=dtype)
+        vc = torch.zeros(nblk, G * Dv, bs, dtype=dtype)
         kc.view(-1, G * P * D)[slots] = k.reshape(n, -1)
-        vc.view(-1, G * Dv)[slots] = v.reshape(n, -1)
+        vc[slots // bs, :, slots % bs] = v.reshape(n, -1)
         rows = [i, min(i + 3, n - 1), j]                          # decode rows ...
         chunk = (i - 5, 9)                                        # ... and a chunk around i
         md = _metadata(device, table, rows, chunk)
@@ -232,7 +234,7 @@ def case_layers(device, dtype, cfg_fn=C.config_a):
         sess.close()
 
 
-def case_schedules(device, dtype, cfg_fn=C.config_a, seed=0):
+def case_schedules(device, dtype, cfg_fn=C.config_a, seed=0, block_size=16):
     """Whole prompts, prompt + one-by-one decoding, portions of several sizes down to two tokens
     and mixed batches with reuse of pages all give the oracle's logits."""
     cfg = cfg_fn()
@@ -241,8 +243,9 @@ def case_schedules(device, dtype, cfg_fn=C.config_a, seed=0):
     reqs = {"a": _tokens(70, V, 11), "b": _tokens(37, V, 12), "c": _tokens(5, V, 13),
             "d": _tokens(1, V, 14), "e": _tokens(49, V, 15)}
     want = {k: C.oracle_logits(cfg, W, t) for k, t in reqs.items()}
-    # pool of 8 pages of 16 tokens: "a" alone needs 5, so pages must be used again
-    sess = C.make_session(cfg, W, device, dtype, max_tokens=128, block_size=16, max_live=2)
+    # pool of 8 pages (of 16 tokens: "a" alone needs 5), so pages must be used again
+    sess = C.make_session(cfg, W, device, dtype, max_tokens=8 * block_size, block_size=block_size,
+                          max_live=2)
     try:
         for k, t in reqs.items():
             got = sess.step([{"id": k, "tokens": t, "want": list(range(len(t)))}], end=[k])
@@ -268,7 +271,8 @@ def case_schedules(device, dtype, cfg_fn=C.config_a, seed=0):
         sess.close()
     # mixed batches on 4 sequences / 10 pages: unequal requests side by side, decode rows beside
     # prompt portions, requests that pause, pages freed and taken again
-    sess = C.make_session(cfg, W, device, dtype, max_tokens=160, block_size=16, max_live=4)
+    sess = C.make_session(cfg, W, device, dtype, max_tokens=10 * block_size, block_size=block_size,
+                          max_live=4)
     try:
         got = {k: [] for k in reqs}
         at = {k: 0 for k in reqs}
