@@ -65,10 +65,15 @@ def parse():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--mode", default="endpoint", choices=["endpoint", "engine", "design"],
-                    help="design: prefill / decode throughput of the Sekolorn design beside a "
-                         "Mixtral-style decoder at equal layer sizes (benchmarks/design_bench.py)")
-    ap.add_argument("--design-sizes", default="s,s6", help="comma list of s, s6 (m, l: gated)")
-    ap.add_argument("--design-models", default="sekolorn,mixtral",
+                    help="design: prefill / decode throughput of a layer-list design beside the "
+                         "closest existing decoder at equal layer sizes (benchmarks/design_bench.py)")
+    ap.add_argument("--design", default="sekolorn", choices=["sekolorn", "vedadra"],
+                    help="design mode: sekolorn beside a Mixtral-style decoder, or vedadra beside "
+                         "a Mistral-style decoder (sliding-window GQA attention + gated MLP)")
+    ap.add_argument("--design-sizes", default=None,
+                    help="comma list; sekolorn: s, s6 (m, l: gated), default s,s6; "
+                         "vedadra: vs, vm, default vs,vm")
+    ap.add_argument("--design-models", default="sekolorn,mixtral,vedadra,mistral",
                     help="which of the two engines to run (profiling one of them alone)")
     ap.add_argument("--design-kernels", action="store_true",
                     help="design mode: time the design's attention / scan kernels beside the "

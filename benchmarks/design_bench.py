@@ -6,6 +6,10 @@ For each size the two engines are built one after the other on the same device:
   with a group-routed ungated MoE and a shared expert;
 * the closest existing family, a Mixtral-style decoder (grouped-query attention + SwiGLU MoE)
   with the same width, layer count, head count, head size, expert count, top-k and expert ff.
+``--design vedadra`` runs the Vedadra design (windowed attention with head mixing, differential
+attention, grouped norms, a looped stack, gated GELU feed-forward) beside a Mistral-style decoder
+(sliding-window grouped-query attention + SwiGLU) with the same width, number of layer runs, head
+count, head size, window and ff.
 Prefill: ``--design-prompts`` prompts of ``--design-prompt-len`` tokens, one sampled token each.
 Decode: ``--design-users`` sequences of 128 prompt tokens generating ``--design-gen`` tokens; the
 decode rate is the extra tokens over the extra time against the same run with one token.
@@ -70,6 +74,35 @@ def mixtral_config(z: dict) -> dict:
             "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "rope_theta": 1e6}
 
 
+VSIZES = {
+    # name: width, layer runs (3 layers looped twice), heads, kv heads, head dim, window, ff, vocab
+    "vs": dict(width=1024, heads=8, kv_heads=2, dim=128, window=1024, ff=4096, vocab=32000),
+    "vm": dict(width=2048, heads=16, kv_heads=4, dim=128, window=1024, ff=8192, vocab=32000),
+}
+
+
+def vedadra_config(z: dict) -> dict:
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                     "mask": {"size": z["window"]}}}
+    att2 = {"type": "attention_2", "mlp": mlp,
+            "mixer": {"heads": H, "kv_heads": G, "dim": D // 2, "vdim": D, "scale": (D // 2) ** -0.5,
+                      "diff": 0.3, "mask": {"size": z["window"], "keep_first": 4}}}
+    return {"architecture": "Vedadra", "vocab": z["vocab"], "width": z["width"],
+            "norm": {"eps": 1e-5, "groups": 4}, "loop": {"start": 0, "stop": 3, "times": 2},
+            "layers": [att, att2, att]}
+
+
+def mistral_config(z: dict) -> dict:
+    return {"architectures": ["MistralForCausalLM"], "hidden_size": z["width"],
+            "num_hidden_layers": 6, "num_attention_heads": z["heads"],
+            "num_key_value_heads": z["kv_heads"], "head_dim": z["dim"], "vocab_size": z["vocab"],
+            "intermediate_size": z["ff"], "sliding_window": z["window"],
+            "max_position_embeddings": 32768, "rms_norm_eps": 1e-5, "rope_theta": 1e6}
+
+
 def _measure(cfg_dict: dict, a) -> dict:
     import torch
 
@@ -119,12 +152,18 @@ def _measure(cfg_dict: dict, a) -> dict:
 
 def run(a) -> int:
     rows = []
-    for name in a.design_sizes.split(","):
+    vedadra = getattr(a, "design", "sekolorn") == "vedadra"
+    for name in (a.design_sizes or ("vs,vm" if vedadra else "s,s6")).split(","):
         if name in GATED:
             raise SystemExit(f"design size {name!r} is switched off (see GATED in "
                              "benchmarks/design_bench.py); run s or s6")
-        z = SIZES[name]
-        for label, cfg in (("Sekolorn", sekolorn_config(z)), ("Mixtral-style", mixtral_config(z))):
+        if vedadra:
+            z = dict(VSIZES[name], layers=6)
+            pair = (("Vedadra", vedadra_config(z)), ("Mistral-style", mistral_config(z)))
+        else:
+            z = SIZES[name]
+            pair = (("Sekolorn", sekolorn_config(z)), ("Mixtral-style", mixtral_config(z)))
+        for label, cfg in pair:
             if label.split("-")[0].lower() not in a.design_models.lower():
                 continue
             r = _measure(cfg, a)
@@ -161,6 +200,8 @@ def kernel_rates(a) -> int:
     (tokens/s and state bytes/s).  One JSON line per kernel."""
     import torch
 
+    if getattr(a, "design", "sekolorn") == "vedadra":
+        return window_kernel_rates(a)
     from enterprise_inference_amd.ops import attention as A
     from enterprise_inference_amd.ops import latent_attention as LA
     from enterprise_inference_amd.ops import wkv as WK
@@ -245,4 +286,114 @@ def kernel_rates(a) -> int:
     for r_ in rows:
         print(json.dumps(r_), flush=True)
     print(json.dumps({"metric": "design_kernel_rates", "rows": rows}), flush=True)
+    return 0
+
+
+def window_kernel_rates(a) -> int:
+    """Achieved rates of the window attention kernels (head-mixing and differential forms) beside
+    the sliding-window paged kernels of the Llama path at equal heads, head size, window and
+    lengths: prefill in useful TFLOP/s (2 P (D + Dv) per visible query-key pair and head; the
+    second product's remainder pass and the head mixing are not counted), decode in cache bytes
+    of the visible keys per second, and the grouped-norm boundary step beside the fused add +
+    RMS norm in bytes moved per second.  One JSON line per kernel."""
+    import torch
+
+    from enterprise_inference_amd.ops import attention as A
+    from enterprise_inference_amd.ops import norm as N
+    from enterprise_inference_amd.ops import window_attention as WA
+
+    dev, bf = "cuda", torch.bfloat16
+    bs, win, T = 128, 1024, 4096
+    rows = []
+    pairs = T * win - win * (win - 1) // 2                     # visible (query, key) pairs
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    for H, G in ((8, 2), (16, 4)):
+        for kind in ("talking", "differential"):
+            P, D, Dv = (1, 128, 128) if kind == "talking" else (2, 64, 128)
+            M = H * P
+            spec = WA.WindowSpec(H, G, P, D, Dv, win, 0 if P == 1 else 4,
+                                 mult=torch.full((M,), D ** -0.5, device=dev))
+            if P == 1:
+                hh = torch.arange(1, H + 1, dtype=torch.float64)
+                spec.slope = torch.pow(2.0, -8.0 * hh / H).float().to(dev)
+                spec.talk = (torch.eye(H) + 0.05 * torch.randn(H, H)).to(dev)
+            else:
+                spec.epilogue, spec.eps, spec.post = 1, 1e-5, 0.7
+                spec.lam = torch.tensor([0.4], device=dev)
+            nb = T // bs
+            kc = torch.randn(nb, bs, G * P * D, device=dev).to(bf)
+            vc = torch.randn(nb, G * Dv, bs, device=dev).to(bf)
+            q = torch.randn(T, M * D, device=dev).to(bf)
+            gate = torch.randn(T, H * Dv, device=dev).to(bf) if P == 1 else None
+            pos = torch.arange(T, dtype=torch.int32, device=dev)
+            bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+            md = A.AttentionMetadata(
+                num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
+                prefill_block_tables=bt, prefill_seq_lens=i32([T]), prefill_cu_q=i32([0, T]),
+                prefill_q_lens=[T])
+            t = _time(lambda: WA.window_attention(q, kc, vc, md, spec, gate))
+            rows.append({"kernel": f"window_attn prefill ({kind})", "heads": H, "kv_heads": G,
+                         "dim": D, "vdim": Dv, "window": win, "tokens": T, "ms": t * 1e3,
+                         "mfma": WA.mfma_ok(spec, bf, bs),
+                         "tflops": 2.0 * P * (D + Dv) * H * pairs / t / 1e12})
+            # decode: B sequences of context L, the last `win` keys visible
+            B, L = 64, 4096
+            nbd = B * L // bs
+            kcd = torch.randn(nbd, bs, G * P * D, device=dev).to(bf)
+            vcd = torch.randn(nbd, G * Dv, bs, device=dev).to(bf)
+            btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
+            posd = torch.full((B,), L - 1, dtype=torch.int32, device=dev)
+            mdd = A.AttentionMetadata(num_decode=B, num_prefill_tokens=0, slot_mapping=posd,
+                                      positions=posd, decode_block_tables=btd,
+                                      decode_seq_lens=i32([L] * B))
+            qd = q[:B].contiguous()
+            gd = gate[:B].contiguous() if gate is not None else None
+            t3 = _time(lambda: WA.window_attention(qd, kcd, vcd, mdd, spec, gd))
+            rows.append({"kernel": f"window_attn decode ({kind})", "heads": H, "kv_heads": G,
+                         "batch": B, "context": L, "window": win, "ms": t3 * 1e3,
+                         "cache_GBps": B * win * G * (P * D + Dv) * 2 / t3 / 1e9})
+        # the like kernels: sliding-window paged prefill (flash form) and decode, D = 128
+        D = 128
+        nb = T // bs
+        kc = torch.randn(nb, G, bs, D, device=dev).to(bf)
+        vc = torch.randn(nb, G, D, bs, device=dev).to(bf)
+        q = torch.randn(T, H, D, device=dev).to(bf) * 0.1
+        bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+        qb2 = A.prefill_query_block(H, G, D, block_size=bs)
+        w2 = A.build_prefill_work([T], qb2)
+        wt = i32(w2)
+        t2 = _time(lambda: A.paged_prefill(q, kc, vc, bt, i32([T]), i32([0, T]), wt, len(w2) // 2,
+                                           0.1, sliding_window=win))
+        rows.append({"kernel": "paged_prefill (flash, sliding window)", "heads": H, "kv_heads": G,
+                     "head_dim": D, "window": win, "tokens": T, "ms": t2 * 1e3,
+                     "tflops": 2.0 * 2 * D * H * pairs / t2 / 1e12})
+        B, L = 64, 4096
+        nbd = B * L // bs
+        kcd = torch.randn(nbd, G, bs, D, device=dev).to(bf)
+        vcd = torch.randn(nbd, G, D, bs, device=dev).to(bf)
+        btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
+        lens = i32([L] * B)
+        qd = q[:B].contiguous()
+        t4 = _time(lambda: A.paged_decode(qd, kcd, vcd, btd, lens, 0.1, sliding_window=win))
+        rows.append({"kernel": "paged_decode (sliding window)", "heads": H, "kv_heads": G,
+                     "batch": B, "context": L, "window": win, "ms": t4 * 1e3,
+                     "cache_GBps": B * win * G * D * 2 * 2 / t4 / 1e9})
+    # sublayer boundary: output norm + residual + next input norm (fp32 stream) beside the
+    # bf16 fused add + RMS norm
+    for W in (2048, 4096):
+        Tn = 8192
+        x = torch.randn(Tn, W, device=dev)
+        y = torch.randn(Tn, W, device=dev).to(bf)
+        w1, w2_ = torch.ones(W, device=dev).to(bf), torch.ones(W, device=dev).to(bf)
+        t5 = _time(lambda: N.group_norm_step(x, 4, 1e-5, y, w1, None, w2_))
+        rows.append({"kernel": "group_norm_step", "width": W, "rows": Tn, "ms": t5 * 1e3,
+                     "GBps": Tn * W * (2 + 4 + 4 + 2) / t5 / 1e9})
+        res = torch.randn(Tn, W, device=dev).to(bf)
+        t6 = _time(lambda: N.fused_add_rms_norm(y, res, w1, 1e-5))
+        rows.append({"kernel": "fused_add_rms_norm", "width": W, "rows": Tn, "ms": t6 * 1e3,
+                     "GBps": Tn * W * (2 + 2 + 2 + 2) / t6 / 1e9})
+    for r_ in rows:
+        print(json.dumps(r_), flush=True)
+    print(json.dumps({"metric": "design_kernel_rates", "design": "vedadra", "rows": rows}),
+          flush=True)
     return 0

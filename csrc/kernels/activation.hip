@@ -109,3 +109,39 @@ EIA_API int eia_relu2(void* out, const void* x, long numel, int is_bf16, hipStre
     hipLaunchKernelGGL(relu2_kernel<float>, grid, block, 0, st, (float*)out, (const float*)x, numel);
   EIA_LAUNCH_CHECK();
 }
+
+// Gated activation straight from the fp32 split-K partials [sk, T, 2F] of a [gate; up] GEMM:
+// out[T, F] = act(sum_z gate_z) * (sum_z up_z), four columns per thread.
+template <int KIND>
+__global__ void __launch_bounds__(256)
+splitk_act_and_mul_kernel(const float* __restrict__ part, int sk, int T, int F,
+                          bf16_t* __restrict__ out, long ldo) {
+  const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= (long)T * F) return;
+  const int row = idx / F, col = idx % F;
+  const long slab = (long)T * 2 * F;
+  const float* p = part + (long)row * 2 * F + col;
+  f32x4 gs = *reinterpret_cast<const f32x4*>(p), us = *reinterpret_cast<const f32x4*>(p + F);
+  for (int z = 1; z < sk; ++z) {
+    gs += *reinterpret_cast<const f32x4*>(p + z * slab);
+    us += *reinterpret_cast<const f32x4*>(p + z * slab + F);
+  }
+  bf16x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = f2bf(act_f<KIND>(gs[i]) * us[i]);
+  *reinterpret_cast<bf16x4*>(out + (long)row * ldo + col) = o;
+}
+
+EIA_API int eia_splitk_act_and_mul(const float* part, int sk, int T, int F, void* out, long ldo,
+                                   int kind, hipStream_t st) {
+  if (F % 4 != 0 || T < 0 || sk < 1 || ldo % 4 != 0) return EIA_BAD_SHAPE;
+  if (T == 0) return EIA_OK;
+  dim3 grid((int)(((long)T * F / 4 + 255) / 256)), block(256);
+  switch (kind) {
+    case ACT_SILU: hipLaunchKernelGGL(splitk_act_and_mul_kernel<ACT_SILU>, grid, block, 0, st, part, sk, T, F, (bf16_t*)out, ldo); break;
+    case ACT_GELU_TANH: hipLaunchKernelGGL(splitk_act_and_mul_kernel<ACT_GELU_TANH>, grid, block, 0, st, part, sk, T, F, (bf16_t*)out, ldo); break;
+    case ACT_GELU_ERF: hipLaunchKernelGGL(splitk_act_and_mul_kernel<ACT_GELU_ERF>, grid, block, 0, st, part, sk, T, F, (bf16_t*)out, ldo); break;
+    default: return EIA_UNSUPPORTED;
+  }
+  EIA_LAUNCH_CHECK();
+}

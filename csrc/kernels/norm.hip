@@ -271,25 +271,39 @@ EIA_API int eia_ln_f32in(const float* x, long ldx, const void* w, void* out, lon
 // lane re-reads only what it wrote and the row needs no barrier.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gnorm_kernel(const T* __restrict__ y, long ldy, const T* __restrict__ w_post,
+gnorm_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ ypart, int sk,
+             long pstride, const T* __restrict__ ybias, const T* __restrict__ w_post,
              float* __restrict__ x, const float* __restrict__ add, const T* __restrict__ w_next,
              T* __restrict__ h, long ldh, float eps, int W, int NG) {
   const long row = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int gs = W / NG;
   float* xr = x + row * (long)W;
+  extern __shared__ float ysum[];                   // [W] when the output arrives as partials
+  if (ypart) {
+    // the whole workgroup sums the GEMM's split-K partials of this row once, into LDS
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      float v = ybias ? ld_f32<T>(ybias, c) : 0.f;
+      const float* p = ypart + row * (long)W + c;
+#pragma unroll 4
+      for (int z = 0; z < sk; ++z) v += p[z * pstride];
+      ysum[c] = v;
+    }
+    __syncthreads();
+  }
+  // the sublayer output at column c: a stored row, or the summed partials
+  auto yval = [&](int c) -> float { return y ? ld_f32<T>(y + row * ldy, c) : ysum[c]; };
   for (int g = wave; g < NG; g += nw) {
     const int c0 = g * gs;
-    if (y) {
-      const T* yr = y + row * ldy + c0;
+    if (y || ypart) {
       float ss = 0.f;
       for (int c = lane; c < gs; c += 64) {
-        const float v = ld_f32<T>(yr, c);
+        const float v = yval(c0 + c);
         ss += v * v;
       }
       const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
       for (int c = lane; c < gs; c += 64)
-        xr[c0 + c] += ld_f32<T>(yr, c) * inv * ld_f32<T>(w_post, c0 + c);
+        xr[c0 + c] += yval(c0 + c) * inv * ld_f32<T>(w_post, c0 + c);
     }
     if (add) {
       const float* ar = add + row * (long)W + c0;
@@ -309,22 +323,29 @@ gnorm_kernel(const T* __restrict__ y, long ldy, const T* __restrict__ w_post,
   }
 }
 
-// x fp32 [rows, W] contiguous, updated in place when y or add is given; y, w_post, w_next, h are
-// bf16 when is_bf16 else fp32.
-EIA_API int eia_gnorm(const void* y, long ldy, const void* w_post, float* x, const float* add,
-                      const void* w_next, void* h, long ldh, float eps, int rows, int W, int NG,
-                      int is_bf16, hipStream_t st) {
-  if (rows < 0 || W < 1 || NG < 1 || W % NG || !x || (y && !w_post) || (h && !w_next))
+// x fp32 [rows, W] contiguous, updated in place when y / ypart or add is given; y, ybias, w_post,
+// w_next, h are bf16 when is_bf16 else fp32.  The sublayer output is either y [rows, W] (row
+// stride ldy) or the fp32 split-K partials ypart [sk, rows, W] of the GEMM that produced it
+// (+ ybias), summed here.
+EIA_API int eia_gnorm(const void* y, long ldy, const float* ypart, int sk, const void* ybias,
+                      const void* w_post, float* x, const float* add, const void* w_next, void* h,
+                      long ldh, float eps, int rows, int W, int NG, int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1 || NG < 1 || W % NG || !x || ((y || ypart) && !w_post) || (h && !w_next) ||
+      (y && ypart) || (ypart && sk < 1))
     return EIA_BAD_SHAPE;
   if (rows == 0) return EIA_OK;
-  const int threads = NG >= 4 ? 256 : 64 * NG;
+  const int threads = (NG >= 4 || ypart) ? 256 : 64 * NG;
+  const long ps = (long)rows * W;
+  const size_t lds = ypart ? sizeof(float) * W : 0;
+  if (lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (is_bf16)
-    hipLaunchKernelGGL((gnorm_kernel<bf16_t>), dim3(rows), dim3(threads), 0, st,
-                       (const bf16_t*)y, ldy, (const bf16_t*)w_post, x, add,
-                       (const bf16_t*)w_next, (bf16_t*)h, ldh, eps, W, NG);
+    hipLaunchKernelGGL((gnorm_kernel<bf16_t>), dim3(rows), dim3(threads), lds, st,
+                       (const bf16_t*)y, ldy, ypart, sk, ps, (const bf16_t*)ybias,
+                       (const bf16_t*)w_post, x, add, (const bf16_t*)w_next, (bf16_t*)h, ldh, eps,
+                       W, NG);
   else
-    hipLaunchKernelGGL((gnorm_kernel<float>), dim3(rows), dim3(threads), 0, st, (const float*)y,
-                       ldy, (const float*)w_post, x, add, (const float*)w_next, (float*)h, ldh,
-                       eps, W, NG);
+    hipLaunchKernelGGL((gnorm_kernel<float>), dim3(rows), dim3(threads), lds, st, (const float*)y,
+                       ldy, ypart, sk, ps, (const float*)ybias, (const float*)w_post, x, add,
+                       (const float*)w_next, (float*)h, ldh, eps, W, NG);
   EIA_LAUNCH_CHECK();
 }

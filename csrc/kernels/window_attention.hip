@@ -27,58 +27,84 @@
 //   q maps  -> RMS norm (weight qw[D]) -> q_out[t, MQ * D]
 //   k maps  -> RMS norm (weight kw[D]) -> key row of the token's slot
 //   values  -> copied as projected     -> value columns of the token's slot (page-transposed)
+//   gate    -> copied as projected     -> gate_out[t, GW]          (GW == 0: no gate columns)
 // (values may alias the un-normed key columns: v_off == k_off).  Slots < 0 write no cache rows.
+// The row is either stored (fused, type T) or still the fp32 split-K partials [sk, T, N] of the
+// projection GEMM (+ bias), summed here; then the gate columns leave in type T for the
+// attention kernel.
 template <typename T>
 __global__ void __launch_bounds__(256)
-qk_norm_cache_kernel(const T* __restrict__ fused, long ld, int q_off, int k_off, int v_off,
-                     int MQ, int MK, int D, int VW, const T* __restrict__ qw,
+qk_norm_cache_kernel(const T* __restrict__ fused, long ld, const float* __restrict__ part, int sk,
+                     long pstride, const T* __restrict__ bias, int q_off, int k_off, int v_off,
+                     int g_off, int MQ, int MK, int D, int VW, int GW, const T* __restrict__ qw,
                      const T* __restrict__ kw, T* __restrict__ q_out, long ldq,
-                     T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots,
-                     int bs, float eps) {
+                     T* __restrict__ kc, T* __restrict__ vc, T* __restrict__ gate_out, long ldg,
+                     const int* __restrict__ slots, int bs, float eps) {
   const long t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  const T* row = fused + t * ld;
   const long slot = slots ? (long)slots[t] : -1;
+  extern __shared__ float rsum[];                   // [ld] when the row arrives as partials
+  if (part) {
+    // the whole workgroup sums the GEMM's split-K partials of this row once, into LDS
+    for (int c = threadIdx.x; c < (int)ld; c += blockDim.x) {
+      float v = bias ? ld_f32<T>(bias, c) : 0.f;
+      const float* p = part + t * ld + c;
+#pragma unroll 4
+      for (int z = 0; z < sk; ++z) v += p[z * pstride];
+      rsum[c] = v;
+    }
+    __syncthreads();
+  }
+  auto val = [&](int c) -> float { return fused ? ld_f32<T>(fused + t * ld, c) : rsum[c]; };
   for (int u = wave; u < MQ + MK; u += nw) {
     const bool isq = u < MQ;
     const int m = isq ? u : u - MQ;
     if (!isq && slot < 0) continue;
-    const T* src = row + (isq ? q_off : k_off) + m * D;
+    const int c0 = (isq ? q_off : k_off) + m * D;
     float ss = 0.f;
     for (int d = lane; d < D; d += 64) {
-      const float v = ld_f32<T>(src, d);
+      const float v = val(c0 + d);
       ss += v * v;
     }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
     T* dst = isq ? q_out + t * ldq + m * D : kc + slot * ((long)MK * D) + m * D;
     const T* w = isq ? qw : kw;
-    for (int d = lane; d < D; d += 64)
-      st_f32<T>(dst, d, ld_f32<T>(src, d) * inv * ld_f32<T>(w, d));
+    for (int d = lane; d < D; d += 64) st_f32<T>(dst, d, val(c0 + d) * inv * ld_f32<T>(w, d));
   }
   if (slot >= 0) {
-    const T* src = row + v_off;
     T* dst = vc + (slot / bs) * (long)VW * bs + slot % bs;
-    for (int c = threadIdx.x; c < VW; c += blockDim.x) dst[(long)c * bs] = src[c];
+    for (int c = threadIdx.x; c < VW; c += blockDim.x) st_f32<T>(dst, (long)c * bs, val(v_off + c));
   }
+  if (gate_out)
+    for (int c = threadIdx.x; c < GW; c += blockDim.x)
+      st_f32<T>(gate_out + t * ldg, c, val(g_off + c));
 }
 
-EIA_API int eia_qk_norm_cache(const void* fused, long ld, int q_off, int k_off, int v_off, int MQ,
-                              int MK, int D, int VW, const void* qw, const void* kw, void* q_out,
-                              long ldq, void* kc, void* vc, const int* slots, int bs, float eps,
-                              int T, int is_bf16, hipStream_t st) {
-  if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || bs < 1 || !fused || !q_out || !kc || !vc)
+EIA_API int eia_qk_norm_cache(const void* fused, long ld, const float* part, int sk,
+                              const void* bias, int q_off, int k_off, int v_off, int g_off, int MQ,
+                              int MK, int D, int VW, int GW, const void* qw, const void* kw,
+                              void* q_out, long ldq, void* kc, void* vc, void* gate_out, long ldg,
+                              const int* slots, int bs, float eps, int T, int is_bf16,
+                              hipStream_t st) {
+  if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || bs < 1 || !q_out || !kc || !vc ||
+      (fused == nullptr) == (part == nullptr) || (part && sk < 1))
     return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
+  const long ps = (long)T * ld;
+  const size_t lds = part ? sizeof(float) * ld : 0;
+  if (lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (is_bf16)
-    hipLaunchKernelGGL((qk_norm_cache_kernel<bf16_t>), dim3(T), dim3(256), 0, st,
-                       (const bf16_t*)fused, ld, q_off, k_off, v_off, MQ, MK, D, VW,
-                       (const bf16_t*)qw, (const bf16_t*)kw, (bf16_t*)q_out, ldq, (bf16_t*)kc,
-                       (bf16_t*)vc, slots, bs, eps);
+    hipLaunchKernelGGL((qk_norm_cache_kernel<bf16_t>), dim3(T), dim3(256), lds, st,
+                       (const bf16_t*)fused, ld, part, sk, ps, (const bf16_t*)bias, q_off, k_off,
+                       v_off, g_off, MQ, MK, D, VW, GW, (const bf16_t*)qw, (const bf16_t*)kw,
+                       (bf16_t*)q_out, ldq, (bf16_t*)kc, (bf16_t*)vc, (bf16_t*)gate_out, ldg, slots,
+                       bs, eps);
   else
-    hipLaunchKernelGGL((qk_norm_cache_kernel<float>), dim3(T), dim3(256), 0, st,
-                       (const float*)fused, ld, q_off, k_off, v_off, MQ, MK, D, VW,
-                       (const float*)qw, (const float*)kw, (float*)q_out, ldq, (float*)kc,
-                       (float*)vc, slots, bs, eps);
+    hipLaunchKernelGGL((qk_norm_cache_kernel<float>), dim3(T), dim3(256), lds, st,
+                       (const float*)fused, ld, part, sk, ps, (const float*)bias, q_off, k_off,
+                       v_off, g_off, MQ, MK, D, VW, GW, (const float*)qw, (const float*)kw,
+                       (float*)q_out, ldq, (float*)kc, (float*)vc, (float*)gate_out, ldg, slots, bs,
+                       eps);
   EIA_LAUNCH_CHECK();
 }
 
@@ -99,6 +125,8 @@ struct WinAttnArgs {
   int H, G, P, D, Dv, bs, window, keep, qb, epilogue;
   const float* lam;                 // [1], epilogue 1
   float eps, post;
+  int nparts;                       // MFMA form: key partitions over grid.z (1: none)
+  float* part_acc; float* part_ml;  // [rows, M, nparts, Dv] and [rows, M, nparts, 2] partials
 };
 
 constexpr int WA_KT = 64;           // keys per tile = lanes of a wave
@@ -279,7 +307,8 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
   if (M * Dv > 256 * WA_ACC || lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
-                out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post};
+                out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post, 1, nullptr,
+                nullptr};
   if (is_bf16)
     hipLaunchKernelGGL((window_attn_kernel<bf16_t>), dim3(n_items), dim3(256), lds, st, a);
   else
@@ -302,10 +331,13 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
 // maps and mixes the rows of its own heads (buffers alternate between blocks).
 // Softmax weights stay fp32: P enters the second product as a bf16 high part plus a bf16
 // remainder, and the normaliser sums the fp32 weights.
-template <int HW, int P, bool TALK, int ND, int NDV>
+template <int HW, int P, bool TALK, bool SHARE, int ND, int NDV>
 __global__ void __launch_bounds__(256)
 window_attn_mfma_kernel(const WinAttnArgs a) {
   constexpr int MW = HW * P;
+  constexpr int NKV = SHARE ? 1 : HW;          // distinct kv heads among this wave's heads
+  constexpr int HPK = HW / NKV;                // heads per kv head
+  constexpr float LOG2E = 1.4426950408889634f;
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -336,6 +368,12 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
       for (int i = lane; i < HW * Dv; i += 64) out[(long)row0 * a.ldo + h0 * Dv + i] = f2bf(0.f);
     return;
   }
+  float* talk_s = lds;                                              // [M, M] (TALK)
+  f32x4* raw_s = reinterpret_cast<f32x4*>(lds + ((M * M + 3) & ~3));  // [2][M][2][64]
+  if constexpr (TALK) {
+    for (int i = threadIdx.x; i < M * M; i += blockDim.x) talk_s[i] = a.talk[i];
+  }
+  const int hs = wave_on ? h0 : 0;                                  // idle waves read head 0
   const bool row_ok = c < nq;
   const long row = row0 + (row_ok ? c : 0);
   const int qpos = a.positions[row];
@@ -347,21 +385,21 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 
   // Q^T operands of this wave's maps: column = query c, rows = d 32 s + 8 g .. + 8
   bf16x8 qf[MW][ND];
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
   for (int m = 0; m < MW; ++m)
 #pragma unroll
     for (int s = 0; s < ND; ++s) {
-      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       const int d = 32 * s + 8 * g;
-      if (wave_on && s < nd && d < D)
-        v = *reinterpret_cast<const bf16x8*>(q + row * a.ldq + (h0 * P + m) * D + d);
-      qf[m][s] = v;
+      const bf16x8 v = *reinterpret_cast<const bf16x8*>(q + row * a.ldq + (hs * P + m) * D +
+                                                        (d < D ? d : 0));
+      qf[m][s] = d < D ? v : zero8;
     }
   float mult[MW], slope[MW];
 #pragma unroll
   for (int m = 0; m < MW; ++m) {
-    mult[m] = wave_on ? a.mult[h0 * P + m] : 0.f;
-    slope[m] = (wave_on && a.slope) ? a.slope[h0 * P + m] : 0.f;
+    mult[m] = a.mult[hs * P + m];
+    slope[m] = a.slope ? a.slope[hs * P + m] : 0.f;
   }
   f32x4 acc[MW][NDV];
   float mrun[MW], lrun[MW];
@@ -372,48 +410,71 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
     for (int t = 0; t < NDV; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
+  // S^T tiles: tile t, row 4 g' + i  <->  key 8 g' + 4 t + i; this lane's A rows are c
+  const int r0 = 8 * (c >> 2) + (c & 3);                            // key of row c in tile 0
+  const int dq = 8 * g;
 
-  for (int b = 0; b < nblocks; ++b) {
+  // with key partitions (decode rows of small batches) this workgroup takes a slice of the blocks
+  const int per = (nblocks + a.nparts - 1) / a.nparts;
+  const int b_lo = blockIdx.z * per, b_hi = min(nblocks, b_lo + per);
+  for (int b = b_lo; b < b_hi; ++b) {
     const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
     const int key0 = kb << 5;
     const long page = bt[key0 / bs];
     const int off = key0 % bs;
-    // S^T tiles: tile t, row 4 g' + i  <->  key 8 g' + 4 t + i; this lane's A rows are c
-    const int r0 = 8 * (c >> 2) + (c & 3);                          // key of row c in tile 0
     const bf16_t* k0p = kc + (page * bs + off + r0) * krow;
-    const bf16_t* k1p = k0p + 4 * krow;
     f32x4 sc[MW][2];
 #pragma unroll
-    for (int m = 0; m < MW; ++m) {
-      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-      if (wave_on) {
-        const int km = (((h0 + m / P) / rep) * P + m % P) * D;
+    for (int j = 0; j < NKV; ++j) {
+      const int kvh = (hs + j * HPK) / rep;
+      // every K operand of this kv head first (addresses clamped, not branched), then the MFMAs
+      bf16x8 kf[P][2][ND];
+#pragma unroll
+      for (int pm = 0; pm < P; ++pm)
 #pragma unroll
         for (int s = 0; s < ND; ++s) {
-          const int d = 32 * s + 8 * g;
-          if (s < nd) {
-            bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb2 = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (d < D) {
-              ka = *reinterpret_cast<const bf16x8*>(k0p + km + d);
-              kb2 = *reinterpret_cast<const bf16x8*>(k1p + km + d);
-            }
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[m][s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb2, qf[m][s], s1, 0, 0, 0);
-          }
+          const int d = 32 * s + dq;
+          const bf16_t* kp = k0p + (kvh * P + pm) * D + (d < D ? d : 0);
+          const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kp);
+          const bf16x8 kb2 = *reinterpret_cast<const bf16x8*>(kp + 4 * krow);
+          kf[pm][0][s] = d < D ? ka : zero8;
+          kf[pm][1][s] = d < D ? kb2 : zero8;
         }
-      }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int ka = key0 + 8 * g + i;
-        s0[i] = s0[i] * mult[m] - slope[m] * (float)(qpos - ka);
-        s1[i] = s1[i] * mult[m] - slope[m] * (float)(qpos - ka - 4);
-      }
-      sc[m][0] = s0;
-      sc[m][1] = s1;
+      for (int hh = 0; hh < HPK; ++hh)
+#pragma unroll
+        for (int pm = 0; pm < P; ++pm) {
+          const int m = (j * HPK + hh) * P + pm;
+          f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < ND; ++s) {
+            if (s < nd) {
+              s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[pm][0][s], qf[m][s], s0, 0, 0, 0);
+              s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[pm][1][s], qf[m][s], s1, 0, 0, 0);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int ka = key0 + 8 * g + i;
+            s0[i] = s0[i] * mult[m] - slope[m] * (float)(qpos - ka);
+            s1[i] = s1[i] * mult[m] - slope[m] * (float)(qpos - ka - 4);
+          }
+          sc[m][0] = s0;
+          sc[m][1] = s1;
+        }
+    }
+    // the block's V^T operands are requested before the softmax arithmetic needs them
+    bf16x8 vf[NKV][NDV];
+#pragma unroll
+    for (int j = 0; j < NKV; ++j) {
+      const bf16_t* vp = vc + page * vpage + ((long)((hs + j * HPK) / rep) * Dv + c) * bs + off + dq;
+#pragma unroll
+      for (int t = 0; t < NDV; ++t)
+        vf[j][t] = *reinterpret_cast<const bf16x8*>(vp + (long)(t < ndv ? t : 0) * 16 * bs);
     }
     if constexpr (TALK) {
       // raw scores of every map through LDS: [buffer][map][tile][lane] f32x4
-      f32x4* buf = reinterpret_cast<f32x4*>(lds) + (size_t)(b & 1) * M * 128;
+      f32x4* buf = raw_s + (size_t)(b & 1) * M * 128;
       if (wave_on) {
 #pragma unroll
         for (int m = 0; m < MW; ++m) {
@@ -422,47 +483,48 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
         }
       }
       __syncthreads();
-      if (wave_on) {
+#pragma unroll
+      for (int m = 0; m < MW; ++m) {
+        sc[m][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+        sc[m][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll 4
+      for (int gm = 0; gm < M; ++gm) {
+        const f32x4 r0v = buf[(gm * 2 + 0) * 64 + lane], r1v = buf[(gm * 2 + 1) * 64 + lane];
 #pragma unroll
         for (int m = 0; m < MW; ++m) {
-          sc[m][0] = f32x4{0.f, 0.f, 0.f, 0.f};
-          sc[m][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-        for (int gm = 0; gm < M; ++gm) {
-          const f32x4 r0v = buf[(gm * 2 + 0) * 64 + lane], r1v = buf[(gm * 2 + 1) * 64 + lane];
-#pragma unroll
-          for (int m = 0; m < MW; ++m) {
-            const float tw = a.talk[(h0 + m) * M + gm];
-            sc[m][0] += tw * r0v;
-            sc[m][1] += tw * r1v;
-          }
+          const float tw = talk_s[(hs + m) * M + gm];
+          sc[m][0] += tw * r0v;
+          sc[m][1] += tw * r1v;
         }
       }
     }
-    if (!wave_on) continue;
     // mask, running max / sum, P^T operands
     bf16x8 ph[MW], pl[MW];
     float alpha[MW];
+    bool vis[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = key0 + 8 * g + e;
+      vis[e] = row_ok && key <= qpos && (a.window <= 0 || qpos - key < a.window || key < a.keep);
+    }
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
       float v[8];
-      bool vis[8];
       float mloc = -1e30f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int key = key0 + 8 * g + e;
-        vis[e] = row_ok && key <= qpos && (a.window <= 0 || qpos - key < a.window || key < a.keep);
         v[e] = e < 4 ? sc[m][0][e] : sc[m][1][e - 4];
         if (vis[e]) mloc = fmaxf(mloc, v[e]);
       }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 16, 64));
       mloc = fmaxf(mloc, __shfl_xor(mloc, 32, 64));
       const float mnew = fmaxf(mrun[m], mloc);
-      alpha[m] = expf(mrun[m] - mnew);
+      alpha[m] = exp2f((mrun[m] - mnew) * LOG2E);
       float psum = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = vis[e] ? expf(v[e] - mnew) : 0.f;
+        const float p = vis[e] ? exp2f((v[e] - mnew) * LOG2E) : 0.f;
         const bf16_t hi = f2bf(p);
         ph[m][e] = hi;
         pl[m][e] = f2bf(p - bf2f(hi));
@@ -475,25 +537,34 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
     }
     // O^T += V^T P^T: A rows = value columns 16 t + c, k = keys 8 g .. + 8 of the block
 #pragma unroll
-    for (int hh = 0; hh < HW; ++hh) {
-      const bf16_t* vp = vc + page * vpage + ((long)((h0 + hh) / rep) * Dv + c) * bs + off + 8 * g;
+    for (int m = 0; m < MW; ++m) {
+      const int j = (m / P) / HPK;
 #pragma unroll
       for (int t = 0; t < NDV; ++t) {
         if (t < ndv) {
-          const bf16x8 vf = *reinterpret_cast<const bf16x8*>(vp + (long)t * 16 * bs);
-#pragma unroll
-          for (int pm = 0; pm < P; ++pm) {
-            const int m = hh * P + pm;
-            f32x4 o = acc[m][t] * alpha[m];
-            o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, ph[m], o, 0, 0, 0);
-            acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[m], o, 0, 0, 0);
-          }
+          f32x4 o = acc[m][t] * alpha[m];
+          o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][t], ph[m], o, 0, 0, 0);
+          acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][t], pl[m], o, 0, 0, 0);
         }
       }
     }
   }
   if (!wave_on || !row_ok) return;
   // this lane holds, per map and tile t, value columns 16 t + 4 g + i of query c
+  if (a.nparts > 1) {                               // partials; window_attn_merge finishes the row
+#pragma unroll
+    for (int m = 0; m < MW; ++m) {
+      const long pr = ((row * M + h0 * P + m) * a.nparts + blockIdx.z);
+      if (g == 0) {
+        a.part_ml[pr * 2] = mrun[m];
+        a.part_ml[pr * 2 + 1] = lrun[m];
+      }
+#pragma unroll
+      for (int t = 0; t < NDV; ++t)
+        if (t < ndv) *reinterpret_cast<f32x4*>(a.part_acc + pr * Dv + 16 * t + 4 * g) = acc[m][t];
+    }
+    return;
+  }
   if (a.epilogue == 0) {
     const bf16_t* gate = (const bf16_t*)a.gate;
 #pragma unroll
@@ -507,7 +578,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             float v = acc[m][t][i] * inv;
-            if (gate) v *= 1.0f / (1.0f + expf(-bf2f(gate[row * a.ldg + col + i])));
+            if (gate) v *= 1.0f / (1.0f + __expf(-bf2f(gate[row * a.ldg + col + i])));
             o[i] = f2bf(v);
           }
           *reinterpret_cast<bf16x4*>(out + row * a.ldo + col) = o;
@@ -544,6 +615,54 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   }
 }
 
+// Merge of key partitions and the row's epilogue: one wave per (row, head).  Lane z first turns
+// partition z's (max, sum) into its weight; the value columns are then summed over the partitions
+// with independent loads (nparts <= 64).
+__global__ void __launch_bounds__(64)
+window_attn_merge_kernel(const WinAttnArgs a) {
+  const int H = a.H, P = a.P, Dv = a.Dv, M = H * P, NP = a.nparts;
+  const long row = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  bf16_t* out = (bf16_t*)a.out + row * a.ldo + h * Dv;
+  if (a.lens && a.lens[row] <= 0) return;           // padding row: the partition kernel wrote zeros
+  float o[2][2];                                    // [map][column lane, lane + 64]
+  for (int pm = 0; pm < P; ++pm) {
+    const long pr = (row * M + h * P + pm) * NP;
+    const float mz = lane < NP ? a.part_ml[(pr + lane) * 2] : -1e30f;
+    const float lz = lane < NP ? a.part_ml[(pr + lane) * 2 + 1] : 0.f;
+    const float wz = __expf(mz - wave_max(mz));
+    const float inv = 1.0f / wave_sum(wz * lz);
+    float v0 = 0.f, v1 = 0.f;
+#pragma unroll 4
+    for (int z = 0; z < NP; ++z) {
+      const float w = __shfl(wz, z, 64);
+      if (lane < Dv) v0 += w * a.part_acc[(pr + z) * Dv + lane];
+      if (lane + 64 < Dv) v1 += w * a.part_acc[(pr + z) * Dv + lane + 64];
+    }
+    o[pm][0] = v0 * inv;
+    o[pm][1] = v1 * inv;
+  }
+  float r0, r1;
+  if (a.epilogue == 0) {
+    const bf16_t* gate = (const bf16_t*)a.gate;
+    r0 = o[0][0];
+    r1 = o[0][1];
+    if (gate) {
+      if (lane < Dv) r0 *= 1.0f / (1.0f + __expf(-bf2f(gate[row * a.ldg + h * Dv + lane])));
+      if (lane + 64 < Dv) r1 *= 1.0f / (1.0f + __expf(-bf2f(gate[row * a.ldg + h * Dv + lane + 64])));
+    }
+  } else {
+    const float lam = a.lam[0];
+    r0 = lane < Dv ? o[0][0] - lam * o[1][0] : 0.f;
+    r1 = lane + 64 < Dv ? o[0][1] - lam * o[1][1] : 0.f;
+    const float inv = a.post / sqrtf(wave_sum(r0 * r0 + r1 * r1) / (float)Dv + a.eps);
+    r0 *= inv;
+    r1 *= inv;
+  }
+  if (lane < Dv) out[lane] = f2bf(r0);
+  if (lane + 64 < Dv) out[lane + 64] = f2bf(r1);
+}
+
 // Heads per wave of the MFMA form for (H, P), 0 when the shape runs the scalar form: with head
 // mixing one workgroup must hold every head (H / HW <= 4 waves); without it the heads are
 // spread over grid.y in workgroups of up to four single-head waves.
@@ -556,9 +675,12 @@ static int wa_mfma_hw(int H, int P, int talk) {
   return 0;
 }
 
-EIA_API int eia_window_attn_mfma_ok(int H, int P, int D, int Dv, int bs, int talk) {
-  return wa_mfma_hw(H, P, talk) > 0 && D % 8 == 0 && D <= 128 && Dv % 16 == 0 && Dv <= 128 &&
-         bs % 32 == 0;
+EIA_API int eia_window_attn_mfma_ok(int H, int G, int P, int D, int Dv, int bs, int talk) {
+  const int hw = wa_mfma_hw(H, P, talk);
+  if (hw == 0 || G < 1 || H % G || D % 8 || D > 128 || Dv % 16 || Dv > 128 || bs % 32) return 0;
+  // four heads of four different kv heads per wave at the large head size would spill
+  if (hw == 4 && (H / G) % 4 != 0 && (D > 64 || Dv > 64)) return 0;
+  return 1;
 }
 
 EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const void* vc,
@@ -567,40 +689,63 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
                                  const float* slope, const float* talk, const void* gate, long ldg,
                                  void* out, long ldo, int H, int G, int P, int D, int Dv, int bs,
                                  int window, int keep, int epilogue, const float* lam, float eps,
-                                 float post, hipStream_t st) {
+                                 float post, int nparts, float* part_acc, float* part_ml,
+                                 hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || bs < 1 || keep < 0 || !q ||
       !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
   if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam))) return EIA_BAD_SHAPE;
-  if (!eia_window_attn_mfma_ok(H, P, D, Dv, bs, talk != nullptr)) return EIA_UNSUPPORTED;
-  if (ldq % 8 || ldo % 4 || (gate && ldg % 1)) return EIA_BAD_SHAPE;
+  if (!eia_window_attn_mfma_ok(H, G, P, D, Dv, bs, talk != nullptr)) return EIA_UNSUPPORTED;
+  if (ldq % 8 || ldo % 4) return EIA_BAD_SHAPE;
+  // key partitions: decode rows only (a row is its own work item), partials in the workspace
+  if (nparts < 1 || nparts > 64 || (nparts > 1 && (cu || !part_acc || !part_ml)))
+    return EIA_BAD_SHAPE;
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
-                out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post};
+                out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post, nparts,
+                part_acc, part_ml};
   const int hw = wa_mfma_hw(H, P, talk != nullptr);
   const int waves_needed = H / hw;
   const int nwv = talk ? waves_needed : (waves_needed < 4 ? waves_needed : 4);
   const int gy = talk ? 1 : (waves_needed + nwv - 1) / nwv;
-  const size_t lds = talk ? (size_t)2 * H * P * 128 * sizeof(f32x4) : 0;
+  const size_t lds = talk ? (size_t)2 * H * P * 128 * sizeof(f32x4) + sizeof(float) * ((H * H + 3) & ~3) : 0;
+  if (lds > 128 * 1024) return EIA_UNSUPPORTED;
+  const bool share = (H / G) % hw == 0;          // the heads of a wave read one kv head
   const bool big = D > 64 || Dv > 64;
-  dim3 grid(n_items, gy), block(64 * nwv);
-#define WA_LAUNCH(HWV, PV, TK)                                                                  \
+  dim3 grid(n_items, gy, nparts), block(64 * nwv);
+#define WA_LAUNCH1(HWV, PV, TK, SH, NDX, NDVX)                                                  \
   do {                                                                                          \
-    if (big)                                                                                    \
-      hipLaunchKernelGGL((window_attn_mfma_kernel<HWV, PV, TK, 4, 8>), grid, block, lds, st, a); \
-    else                                                                                        \
-      hipLaunchKernelGGL((window_attn_mfma_kernel<HWV, PV, TK, 2, 4>), grid, block, lds, st, a); \
+    if (lds > 48 * 1024)                                                                        \
+      (void)hipFuncSetAttribute(                                                                \
+          reinterpret_cast<const void*>(&window_attn_mfma_kernel<HWV, PV, TK, SH, NDX, NDVX>),  \
+          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                \
+    hipLaunchKernelGGL((window_attn_mfma_kernel<HWV, PV, TK, SH, NDX, NDVX>), grid, block, lds, \
+                       st, a);                                                                  \
   } while (0)
+#define WA_LAUNCH(HWV, PV, TK, SH)                                                              \
+  do {                                                                                          \
+    if (big) WA_LAUNCH1(HWV, PV, TK, SH, 4, 8);                                                 \
+    else WA_LAUNCH1(HWV, PV, TK, SH, 2, 4);                                                     \
+  } while (0)
+  // without head mixing the key width may be half the value width (a differential pair)
+  const bool narrow_k = !talk && D <= 64 && Dv > 64;
   if (talk) {
-    if (hw == 1) WA_LAUNCH(1, 1, true);
-    else if (hw == 2) WA_LAUNCH(2, 1, true);
-    else WA_LAUNCH(4, 1, true);
+    if (hw == 1) WA_LAUNCH(1, 1, true, true);
+    else if (hw == 2 && share) WA_LAUNCH(2, 1, true, true);
+    else if (hw == 2) WA_LAUNCH(2, 1, true, false);
+    else if (share) WA_LAUNCH(4, 1, true, true);
+    else WA_LAUNCH1(4, 1, true, false, 2, 4);
   } else if (P == 2) {
-    WA_LAUNCH(1, 2, false);
+    if (narrow_k) WA_LAUNCH1(1, 2, false, true, 2, 8);
+    else WA_LAUNCH(1, 2, false, true);
   } else {
-    WA_LAUNCH(1, 1, false);
+    if (narrow_k) WA_LAUNCH1(1, 1, false, true, 2, 8);
+    else WA_LAUNCH(1, 1, false, true);
   }
 #undef WA_LAUNCH
+#undef WA_LAUNCH1
+  if (nparts > 1)
+    hipLaunchKernelGGL(window_attn_merge_kernel, dim3(n_items, H), dim3(64), 0, st, a);
   EIA_LAUNCH_CHECK();
 }

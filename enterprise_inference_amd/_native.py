@@ -77,13 +77,15 @@ _SIGNATURES = {
     "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, I, S],
     "eia_relu2": [P, P, L, I, S],
     "eia_moe_combine_postnorm": [P, L, P, P, I, P, L, P, F, P, P, L, I, I, I, S],
-    "eia_gnorm": [P, L, P, P, P, P, P, L, F, I, I, I, I, S],
-    "eia_qk_norm_cache": [P, L, I, I, I, I, I, I, I, P, P, P, L, P, P, IP, I, F, I, I, S],
+    "eia_gnorm": [P, L, P, I, P, P, P, P, P, P, L, F, I, I, I, I, S],
+    "eia_splitk_act_and_mul": [P, I, I, I, P, L, I, S],
+    "eia_qk_norm_cache": [P, L, P, I, P, I, I, I, I, I, I, I, I, I, P, P, P, L, P, P, P, L, IP, I, F,
+                          I, I, S],
     "eia_window_attn": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I, I,
                         I, I, I, I, I, P, F, F, I, S],
     "eia_window_attn_mfma": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I,
-                             I, I, I, I, I, P, F, F, S],
-    "eia_window_attn_mfma_ok": [I, I, I, I, I, I],
+                             I, I, I, I, I, P, F, F, I, P, P, S],
+    "eia_window_attn_mfma_ok": [I, I, I, I, I, I, I],
     "eia_ar_alloc": [P, L],
     "eia_moe_splitk_norm_route": [P, I, I, I, P, P, F, P, L, P, I, I, I, I, P, P, P, S],
     "eia_moe_combine_norm": [P, I, I, P, P, I, I, I, P, P, F, P, L, S],

@@ -93,6 +93,10 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
                 x.dim() == 2 and gemm.skinny_ok(x, self.weight, swiglu=True):
             return gemm.swiglu_gemm(x, self.weight)
         from ..ops import activation
+        if self.bias is None and x.dim() == 2:
+            # other activations: a decode-sized GEMM's split-K partials are summed inside the
+            # activation kernel
+            return activation.act_and_mul(gemm.linear(x, self.weight, None, defer_reduce=True), act)
         return activation.act_and_mul(gemm.linear(x, self.weight, self.bias), act)
 
 

@@ -245,16 +245,16 @@ class _WindowMixerBase(nn.Module):
         pass
 
     def _attend(self, xb, md, cache: PagedKVRows, v_part: str, gate_part=None):
-        fused = gemm.linear(xb, self.proj, self.proj_bias)
+        # decode-sized batches: the projection's split-K partials go straight to the cache-write
+        # kernel, which sums them (no separate reduce launch, no bf16 round trip)
+        fused = gemm.linear(xb, self.proj, self.proj_bias, defer_reduce=True)
         P = self.maps
-        q = win_ops.qk_norm_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
-                                  self.offsets[v_part][0], self.heads * P, self.kv_heads * P,
-                                  self.dim, self.kv_heads * self.vdim, self.q_norm, self.k_norm,
-                                  cache.k, cache.v, md.slot_mapping, self.eps)
-        gate = None
-        if gate_part is not None:
-            g0, gn = self.offsets[gate_part]
-            gate = fused[:, g0:g0 + gn]
+        g0, gn = self.offsets[gate_part] if gate_part is not None else (0, 0)
+        q, gate = win_ops.qk_norm_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
+                                        self.offsets[v_part][0], self.heads * P, self.kv_heads * P,
+                                        self.dim, self.kv_heads * self.vdim, self.q_norm,
+                                        self.k_norm, cache.k, cache.v, md.slot_mapping, self.eps,
+                                        g0, gn)
         return win_ops.window_attention(q, cache.k, cache.v, md, self.spec, gate)
 
 
@@ -284,7 +284,9 @@ class TalkingWindowAttentionMixer(_WindowMixerBase):
         self.spec.talk.copy_(self.talk.float())
 
     def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
-        return gemm.linear(self._attend(xb, md, cache, "k", "g"), self.o, self.o_bias)
+        # may return gemm.SplitK: the output norm step reduces it
+        return gemm.linear(self._attend(xb, md, cache, "k", "g"), self.o, self.o_bias,
+                           defer_reduce=True)
 
 
 class DifferentialAttentionMixer(_WindowMixerBase):
@@ -314,4 +316,4 @@ class DifferentialAttentionMixer(_WindowMixerBase):
         self.spec.lam.copy_((a - b + self.diff).reshape(1))
 
     def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
-        return gemm.linear(self._attend(xb, md, cache, "v"), self.o)
+        return gemm.linear(self._attend(xb, md, cache, "v"), self.o, defer_reduce=True)

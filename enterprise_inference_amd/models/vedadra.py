@@ -79,7 +79,8 @@ class VedadraLayer(nn.Module):
         if self.mlp is None:
             return norm_ops.group_norm_step(x, self.groups, self.eps, y, self.norm1b, add, w_next)
         h = norm_ops.group_norm_step(x, self.groups, self.eps, y, self.norm1b, None, self.norm2)
-        y = self.mlp.down_proj(self.mlp.gate_up_proj.forward_act_and_mul(h, self.mlp.act))
+        y = self.mlp.down_proj(self.mlp.gate_up_proj.forward_act_and_mul(h, self.mlp.act),
+                               defer_reduce=True)
         return norm_ops.group_norm_step(x, self.groups, self.eps, y, self.norm2b, add, w_next)
 
 

@@ -11,8 +11,19 @@ _KIND = {"silu": 0, "swiglu": 0, "gelu_tanh": 1, "gelu_pytorch_tanh": 1, "gelu_n
          "gelu": 2, "gelu_erf": 2}
 
 
-def act_and_mul(x: torch.Tensor, act: str = "silu") -> torch.Tensor:
+def act_and_mul(x, act: str = "silu") -> torch.Tensor:
+    """act(x[:, :F]) * x[:, F:].  x may be a ``gemm.SplitK`` (fp32 partial sums of the [gate; up]
+    GEMM): they are then summed inside the activation kernel."""
+    from .gemm import SplitK
     kind = _KIND[act]
+    if isinstance(x, SplitK):
+        F = x.N // 2
+        if x.bias is None and x.part.is_cuda and x.part.is_contiguous() and F % 4 == 0:
+            out = torch.empty((x.M, F), dtype=torch.bfloat16, device=x.part.device)
+            check(lib().eia_splitk_act_and_mul(ptr(x.part), x.sk, x.M, F, ptr(out), out.stride(0),
+                                               kind, stream(out)), "splitk_act_and_mul")
+            return out
+        x = x.materialize()
     if not (use_hip(x) and x.dtype == torch.bfloat16):
         return ref.silu_and_mul(x) if kind == 0 else ref.gelu_and_mul(x) if kind == 1 else (
             (torch.nn.functional.gelu(x[..., :x.shape[-1] // 2].float()) *

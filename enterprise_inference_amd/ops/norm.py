@@ -107,7 +107,7 @@ def _group_rms(v: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
     return (p / torch.sqrt((p * p).mean(-1, keepdim=True) + eps)).reshape(v.shape)
 
 
-def group_norm_step(x: torch.Tensor, groups: int, eps: float, y: Optional[torch.Tensor] = None,
+def group_norm_step(x: torch.Tensor, groups: int, eps: float, y=None,
                     w_post: Optional[torch.Tensor] = None, add: Optional[torch.Tensor] = None,
                     w_next: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """One sublayer boundary of a model whose norms are RMS norms in ``groups`` equal consecutive
@@ -118,10 +118,16 @@ def group_norm_step(x: torch.Tensor, groups: int, eps: float, y: Optional[torch.
         x += add                    (add given: fp32 rows, in place)
         h  = gnorm(x) * w_next      (w_next given: returned in the weights' dtype)
 
-    All arithmetic is fp32; y and the weights are in the activation dtype."""
+    All arithmetic is fp32; y and the weights are in the activation dtype.  y may also be a
+    ``gemm.SplitK`` (the fp32 partial sums of the GEMM that produced it, plus its bias): the
+    reduction then happens here, on fp32 values that were never rounded."""
+    from .gemm import SplitK
     T, W = x.shape
     require(W % groups == 0, "group_norm_step: width not divisible by the group count")
+    split = isinstance(y, SplitK)
     if not use_hip(x):
+        if split:
+            y = y.part.sum(0) + (y.bias.float() if y.bias is not None else 0.0)
         if y is not None:
             x += _group_rms(y.float(), groups, eps) * w_post.float()
         if add is not None:
@@ -134,9 +140,17 @@ def group_norm_step(x: torch.Tensor, groups: int, eps: float, y: Optional[torch.
     require(ref_w is not None and ref_w.dtype in (torch.bfloat16, torch.float32),
             "group_norm_step: bf16 or fp32 weights")
     bf = ref_w.dtype == torch.bfloat16
-    if y is not None:
+    part = ybias = yt = None
+    sk = 0
+    if split:
+        require(y.M == T and y.N == W and y.part.is_contiguous() and y.part.dtype == torch.float32
+                and w_post is not None and w_post.dtype == ref_w.dtype and w_post.numel() == W
+                and (y.bias is None or y.bias.dtype == ref_w.dtype), "group_norm_step: partials")
+        part, sk, ybias = y.part, y.sk, y.bias
+    elif y is not None:
         require(y.shape == x.shape and y.stride(-1) == 1 and y.dtype == ref_w.dtype and
                 w_post.dtype == ref_w.dtype and w_post.numel() == W, "group_norm_step: y layout")
+        yt = y
     if add is not None:
         require(add.dtype == torch.float32 and add.is_contiguous() and add.shape == x.shape,
                 "group_norm_step: add layout")
@@ -144,7 +158,7 @@ def group_norm_step(x: torch.Tensor, groups: int, eps: float, y: Optional[torch.
     if w_next is not None:
         require(w_next.numel() == W, "group_norm_step: weight size")
         h = torch.empty(T, W, dtype=w_next.dtype, device=x.device)
-    check(lib().eia_gnorm(ptr(y), y.stride(0) if y is not None else 0, ptr(w_post), ptr(x),
-                          ptr(add), ptr(w_next), ptr(h), W, float(eps), T, W, groups,
-                          1 if bf else 0, stream(x)), "gnorm")
+    check(lib().eia_gnorm(ptr(yt), yt.stride(0) if yt is not None else 0, ptr(part), sk,
+                          ptr(ybias), ptr(w_post), ptr(x), ptr(add), ptr(w_next), ptr(h), W,
+                          float(eps), T, W, groups, 1 if bf else 0, stream(x)), "gnorm")
     return h

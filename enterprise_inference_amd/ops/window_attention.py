@@ -60,12 +60,33 @@ def build_work(q_lens: List[int], qblock: int) -> List[int]:
 
 def mfma_ok(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> bool:
     """The MFMA kernel takes bf16 rows with D % 8 == 0, Dv % 16 == 0, both <= 128, pages of a
-    multiple of 32 tokens and, with head mixing, at most 16 heads in 1, 2 or 4 heads per wave;
-    everything else (fp32 models too) runs the scalar-FMA kernel."""
+    multiple of 32 tokens and, with head mixing, at most 16 heads in 1, 2 or 4 heads per wave
+    (four heads of four different kv heads only up to head size 64); everything else (fp32
+    models too) runs the scalar-FMA kernel."""
     if dtype != torch.bfloat16 or not _MFMA_ENV or not torch.cuda.is_available():
         return False
-    return bool(lib().eia_window_attn_mfma_ok(spec.heads, spec.maps, spec.dim, spec.vdim,
+    return bool(lib().eia_window_attn_mfma_ok(spec.heads, spec.kv_heads, spec.maps, spec.dim,
+                                              spec.vdim,
                                               block_size, 1 if spec.talk is not None else 0))
+
+
+def decode_partitions(batch: int, spec: WindowSpec, cus: int = 256) -> int:
+    """Key partitions (grid.z) of a decode launch of the MFMA form: a decode row is one
+    workgroup (per four heads without head mixing), so small batches split every row's 32-key
+    blocks until about two workgroups per CU exist (a power of two, at most 8, and at least
+    four blocks of a full window per partition); a second kernel merges the partials.  Depends on the
+    batch and the layer's constants only, so a captured decode graph keeps its grid."""
+    forced = int(os.environ.get("EIA_WINDOW_DECODE_P", "0"))
+    if forced > 0:
+        return min(forced, 64)
+    wgs = max(1, batch) * (1 if spec.talk is not None else -(-spec.heads // 4))
+    limit = 8
+    if spec.window > 0:
+        limit = max(1, min(8, ((spec.window + 31) // 32 + 1 + (spec.keep + 31) // 32) // 4))
+    p = 1
+    while p * 2 <= limit and wgs * p * 2 <= 2 * cus:
+        p *= 2
+    return p
 
 
 def query_block(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> int:
@@ -76,17 +97,26 @@ def _rms(v: torch.Tensor, eps: float) -> torch.Tensor:
     return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
 
 
-def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: int, mk: int,
+def qk_norm_cache(fused, q_off: int, k_off: int, v_off: int, mq: int, mk: int,
                   dim: int, v_width: int, q_w: torch.Tensor, k_w: torch.Tensor,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
-                  eps: float) -> torch.Tensor:
+                  eps: float, gate_off: int = 0, gate_width: int = 0):
     """One pass over fused projection rows [T, *]: the ``mq`` query maps at ``q_off`` are
     RMS-normed (weight ``q_w`` [dim]) and returned [T, mq*dim]; the ``mk`` key maps at ``k_off``
     are RMS-normed (``k_w``) into the token's key row and the ``v_width`` value columns at
-    ``v_off`` (which may be the un-normed key columns) are copied into its value row.  Rows with
-    a slot < 0 write no cache."""
-    T = fused.shape[0]
-    if not use_hip(fused):
+    ``v_off`` (which may be the un-normed key columns) are copied into its value columns.  Rows
+    with a slot < 0 write no cache.  Returns (q, gate): gate is the ``gate_width`` columns at
+    ``gate_off`` (None when the width is 0).  ``fused`` may be a ``gemm.SplitK``: the projection's
+    fp32 partial sums (+ bias) are then reduced here and the gate columns written out."""
+    from .gemm import SplitK
+    split = isinstance(fused, SplitK)
+    if split and not fused.part.is_cuda:            # CPU path: the plain fp32 sum
+        fused = fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
+        split = False
+    if not split:
+        T = fused.shape[0]
+        gate = fused[:, gate_off:gate_off + gate_width] if gate_width else None
+    if not split and not use_hip(fused):
         f = fused.float()
         q = _rms(f[:, q_off:q_off + mq * dim].reshape(T, mq, dim), eps) * q_w.float()
         k = _rms(f[:, k_off:k_off + mk * dim].reshape(T, mk, dim), eps) * k_w.float()
@@ -95,26 +125,40 @@ def qk_norm_cache(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, mq: i
         k_cache.view(-1, k_cache.shape[-1])[sm[ok]] = k.reshape(T, -1)[ok].to(k_cache.dtype)
         bs = v_cache.shape[2]
         v_cache[sm[ok] // bs, :, sm[ok] % bs] = fused[:, v_off:v_off + v_width][ok].to(v_cache.dtype)
-        return q.reshape(T, mq * dim).to(fused.dtype)
-    bf = fused.dtype == torch.bfloat16
-    require(bf or fused.dtype == torch.float32, "qk_norm_cache: bf16 or fp32")
-    require(fused.stride(1) == 1 and max(q_off + mq * dim, k_off + mk * dim, v_off + v_width)
-            <= fused.shape[1], "qk_norm_cache: fused row layout")
-    require(k_cache.dtype == fused.dtype and v_cache.dtype == fused.dtype and
-            k_cache.is_contiguous() and v_cache.is_contiguous() and
+        return q.reshape(T, mq * dim).to(fused.dtype), gate
+    dt = k_cache.dtype
+    bf = dt == torch.bfloat16
+    require(bf or dt == torch.float32, "qk_norm_cache: bf16 or fp32")
+    if split:
+        T, width = fused.M, fused.N
+        require(fused.part.dtype == torch.float32 and fused.part.is_contiguous() and
+                (fused.bias is None or fused.bias.dtype == dt), "qk_norm_cache: partials")
+    else:
+        width = fused.shape[1]
+        require(fused.stride(1) == 1 and fused.dtype == dt, "qk_norm_cache: fused row layout")
+    require(max(q_off + mq * dim, k_off + mk * dim, v_off + v_width, gate_off + gate_width)
+            <= width, "qk_norm_cache: columns outside the row")
+    require(v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
             k_cache.shape[-1] == mk * dim and v_cache.shape[1] == v_width and
-            v_cache.shape[2] == k_cache.shape[1],
-            "qk_norm_cache: cache layout")
-    require(q_w.dtype == fused.dtype and k_w.dtype == fused.dtype and q_w.numel() == dim and
-            k_w.numel() == dim, "qk_norm_cache: norm weights")
+            v_cache.shape[2] == k_cache.shape[1], "qk_norm_cache: cache layout")
+    require(q_w.dtype == dt and k_w.dtype == dt and q_w.numel() == dim and k_w.numel() == dim,
+            "qk_norm_cache: norm weights")
     require(slot_mapping.dtype == torch.int32 and slot_mapping.numel() >= T, "int32 slots")
-    q = torch.empty(T, mq * dim, dtype=fused.dtype, device=fused.device)
-    check(lib().eia_qk_norm_cache(ptr(fused), fused.stride(0), q_off, k_off, v_off, mq, mk, dim,
-                                  v_width, ptr(q_w), ptr(k_w), ptr(q), q.stride(0), ptr(k_cache),
-                                  ptr(v_cache), ptr(slot_mapping), k_cache.shape[1], float(eps), T,
-                                  1 if bf else 0,
-                                  stream(fused)), "qk_norm_cache")
-    return q
+    q = torch.empty(T, mq * dim, dtype=dt, device=k_cache.device)
+    if split:
+        gate = torch.empty(T, gate_width, dtype=dt, device=q.device) if gate_width else None
+        check(lib().eia_qk_norm_cache(
+            None, width, ptr(fused.part), fused.sk, ptr(fused.bias), q_off, k_off, v_off, gate_off,
+            mq, mk, dim, v_width, gate_width, ptr(q_w), ptr(k_w), ptr(q), q.stride(0),
+            ptr(k_cache), ptr(v_cache), ptr(gate), gate_width, ptr(slot_mapping),
+            k_cache.shape[1], float(eps), T, 1 if bf else 0, stream(q)), "qk_norm_cache")
+        return q, gate
+    check(lib().eia_qk_norm_cache(
+        ptr(fused), fused.stride(0), None, 0, None, q_off, k_off, v_off, 0, mq, mk, dim, v_width,
+        0, ptr(q_w), ptr(k_w), ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), None, 0,
+        ptr(slot_mapping), k_cache.shape[1], float(eps), T, 1 if bf else 0, stream(q)),
+        "qk_norm_cache")
+    return q, gate
 
 
 def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpec, seq_of_row):
@@ -194,13 +238,18 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         qa, o = q[lo:], out[lo:]
         g = None if gate is None else gate[lo:]
         if mfma:
+            NP = decode_partitions(n_items, spec) if cu is None else 1
+            pa = pm = None
+            if NP > 1:
+                pa = torch.empty(n_items * H * P * NP * Dv, dtype=torch.float32, device=q.device)
+                pm = torch.empty(n_items * H * P * NP * 2, dtype=torch.float32, device=q.device)
             check(lib().eia_window_attn_mfma(
                 ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
                 ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
                 ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0,
                 ptr(o), o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep,
-                spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), stream(q)),
-                "window_attn_mfma")
+                spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), NP, ptr(pa),
+                ptr(pm), stream(q)), "window_attn_mfma")
             return
         check(lib().eia_window_attn(
             ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),

@@ -38,13 +38,20 @@ def _np(t):
 # ------------------------------------------------------------------ mechanisms alone
 def case_group_norm(device, dtype):
     """Every combination of the sublayer-boundary step: output norm + residual, added rows,
-    next input norm; group counts 1, 3, 4 and one group per pair of columns."""
+    next input norm; group counts 1, 3, 4 and one group per pair of columns; the sublayer output
+    as a stored row (use_y 1) or as the split-K partial sums of its GEMM plus a bias (use_y 2)."""
     from enterprise_inference_amd.ops import norm
+    from enterprise_inference_amd.ops.gemm import SplitK
     g = torch.Generator().manual_seed(1)
     for W, groups in ((48, 3), (40, 1), (256, 4), (64, 32), (130, 2)):
-        for use_y, use_add, use_next in ((1, 0, 1), (1, 1, 1), (0, 0, 1), (0, 1, 1), (1, 0, 0)):
+        for use_y, use_add, use_next in ((1, 0, 1), (1, 1, 1), (0, 0, 1), (0, 1, 1), (1, 0, 0),
+                                         (2, 0, 1), (2, 1, 0)):
             x = torch.randn(5, W, generator=g) * 2
             y = (torch.randn(5, W, generator=g) * 3 + 0.5).to(dtype)
+            part = torch.randn(3, 5, W, generator=g) * 2
+            bias = torch.randn(W, generator=g).to(dtype)
+            if use_y == 2:
+                y = part.double().sum(0) + bias.double()
             add = torch.randn(5, W, generator=g)
             w1 = torch.randn(W, generator=g).to(dtype)
             w2 = torch.randn(W, generator=g).to(dtype)
@@ -58,7 +65,11 @@ def case_group_norm(device, dtype):
                 want_x.append(v)
                 want_h.append(O.group_norm(v, _np(w2), groups, 1e-5))
             xd = x.clone().to(device)
-            h = norm.group_norm_step(xd, groups, 1e-5, y.to(device) if use_y else None,
+            if use_y == 2:
+                y_in = SplitK(part.to(device), 3, 5, W, bias.to(device))
+            else:
+                y_in = y.to(device) if use_y else None
+            h = norm.group_norm_step(xd, groups, 1e-5, y_in,
                                      w1.to(device) if use_y else None,
                                      add.to(device) if use_add else None,
                                      w2.to(device) if use_next else None)
@@ -74,23 +85,29 @@ def case_qk_norm_cache(device, dtype):
     """Per-map RMS norm of queries and keys, values copied as projected (also when they are the
     un-normed key columns), rows without a slot skipped, other slots untouched."""
     from enterprise_inference_amd.ops import window_attention as wa
+    from enterprise_inference_amd.ops.gemm import SplitK
     g = torch.Generator().manual_seed(2)
-    for mq, mk, D, vw, alias in ((4, 2, 16, 32, True), (6, 2, 10, 14, False), (2, 2, 96, 40, False),
-                                 (1, 1, 5, 5, True)):
+    for mq, mk, D, vw, alias, split in ((4, 2, 16, 32, True, 0), (6, 2, 10, 14, False, 0),
+                                        (2, 2, 96, 40, False, 0), (1, 1, 5, 5, True, 0),
+                                        (4, 2, 16, 32, True, 3), (3, 1, 24, 20, False, 2)):
         T, bs, nb = 7, 4, 5
         k_off, q_off = 3, 3 + mk * D + (0 if alias else vw)
         v_off = k_off if alias else k_off + mk * D
         width = q_off + mq * D + 2
         fused = (torch.randn(T, width, generator=g) * 2).to(dtype)
+        part = torch.randn(max(split, 1), T, width, generator=g)
+        bias = torch.randn(width, generator=g).to(dtype)
         qw = (1 + 0.3 * torch.randn(D, generator=g)).to(dtype)
         kw = (1 + 0.3 * torch.randn(D, generator=g)).to(dtype)
         slots = torch.tensor([9, 2, -1, 17, 0, 5, 19], dtype=torch.int32)
         kc = torch.full((nb, bs, mk * D), 7.0, dtype=dtype)
         vc = torch.full((nb, vw, bs), 7.0, dtype=dtype)
         kd, vd = kc.to(device), vc.to(device)
-        q = wa.qk_norm_cache(fused.to(device), q_off, k_off, v_off, mq, mk, D, vw, qw.to(device),
-                             kw.to(device), kd, vd, slots.to(device), 1e-5)
-        f = _np(fused)
+        src = SplitK(part.to(device), split, T, width, bias.to(device)) if split else fused.to(device)
+        q, gate = wa.qk_norm_cache(src, q_off, k_off, v_off, mq, mk, D, vw, qw.to(device),
+                                   kw.to(device), kd, vd, slots.to(device), 1e-5, 1, 3)
+        f = (part.double().sum(0) + bias.double()).numpy() if split else _np(fused)
+        assert np.allclose(_np(gate), f[:, 1:4], atol=ktol(dtype), rtol=ktol(dtype))
         for t in range(T):
             for m in range(mq):
                 want = O.rms_div(f[t, q_off + m * D:q_off + (m + 1) * D], 1e-5) * _np(qw)
@@ -105,7 +122,8 @@ def case_qk_norm_cache(device, dtype):
             for m in range(mk):
                 want = O.rms_div(f[t, k_off + m * D:k_off + (m + 1) * D], 1e-5) * _np(kw)
                 assert np.allclose(kflat[s, m * D:(m + 1) * D], want, atol=ktol(dtype), rtol=ktol(dtype))
-            assert np.array_equal(vflat[s], f[t, v_off:v_off + vw])
+            assert np.allclose(vflat[s], f[t, v_off:v_off + vw], atol=ktol(dtype) if split else 0,
+                               rtol=ktol(dtype) if split else 0)
         for s in range(nb * bs):
             if s not in used:
                 assert (kflat[s] == 7.0).all() and (vflat[s] == 7.0).all()
