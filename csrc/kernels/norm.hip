@@ -282,12 +282,15 @@ gnorm_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ ypart,
   extern __shared__ float ysum[];                   // [W] when the output arrives as partials
   if (ypart) {
     // the whole workgroup sums the GEMM's split-K partials of this row once, into LDS
-    for (int c = threadIdx.x; c < W; c += blockDim.x) {
-      float v = ybias ? ld_f32<T>(ybias, c) : 0.f;
+    // (16-byte loads, eight partials in flight per thread; W % 4 == 0)
+    for (int c = 4 * threadIdx.x; c < W; c += 4 * blockDim.x) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (ybias) v = f32x4{ld_f32<T>(ybias, c), ld_f32<T>(ybias, c + 1), ld_f32<T>(ybias, c + 2),
+                           ld_f32<T>(ybias, c + 3)};
       const float* p = ypart + row * (long)W + c;
-#pragma unroll 4
-      for (int z = 0; z < sk; ++z) v += p[z * pstride];
-      ysum[c] = v;
+#pragma unroll 8
+      for (int z = 0; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * pstride);
+      *reinterpret_cast<f32x4*>(ysum + c) = v;
     }
     __syncthreads();
   }
@@ -331,7 +334,7 @@ EIA_API int eia_gnorm(const void* y, long ldy, const float* ypart, int sk, const
                       const void* w_post, float* x, const float* add, const void* w_next, void* h,
                       long ldh, float eps, int rows, int W, int NG, int is_bf16, hipStream_t st) {
   if (rows < 0 || W < 1 || NG < 1 || W % NG || !x || ((y || ypart) && !w_post) || (h && !w_next) ||
-      (y && ypart) || (ypart && sk < 1))
+      (y && ypart) || (ypart && (sk < 1 || W % 4)))
     return EIA_BAD_SHAPE;
   if (rows == 0) return EIA_OK;
   const int threads = (NG >= 4 || ypart) ? 256 : 64 * NG;

@@ -46,12 +46,15 @@ qk_norm_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
   extern __shared__ float rsum[];                   // [ld] when the row arrives as partials
   if (part) {
     // the whole workgroup sums the GEMM's split-K partials of this row once, into LDS
-    for (int c = threadIdx.x; c < (int)ld; c += blockDim.x) {
-      float v = bias ? ld_f32<T>(bias, c) : 0.f;
+    // (16-byte loads, eight partials in flight per thread; ld % 4 == 0)
+    for (int c = 4 * threadIdx.x; c < (int)ld; c += 4 * blockDim.x) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (bias) v = f32x4{ld_f32<T>(bias, c), ld_f32<T>(bias, c + 1), ld_f32<T>(bias, c + 2),
+                          ld_f32<T>(bias, c + 3)};
       const float* p = part + t * ld + c;
-#pragma unroll 4
-      for (int z = 0; z < sk; ++z) v += p[z * pstride];
-      rsum[c] = v;
+#pragma unroll 8
+      for (int z = 0; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * pstride);
+      *reinterpret_cast<f32x4*>(rsum + c) = v;
     }
     __syncthreads();
   }
@@ -87,7 +90,7 @@ EIA_API int eia_qk_norm_cache(const void* fused, long ld, const float* part, int
                               const int* slots, int bs, float eps, int T, int is_bf16,
                               hipStream_t st) {
   if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || bs < 1 || !q_out || !kc || !vc ||
-      (fused == nullptr) == (part == nullptr) || (part && sk < 1))
+      (fused == nullptr) == (part == nullptr) || (part && (sk < 1 || ld % 4)))
     return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
   const long ps = (long)T * ld;
@@ -128,6 +131,19 @@ struct WinAttnArgs {
   int nparts;                       // MFMA form: key partitions over grid.z (1: none)
   float* part_acc; float* part_ml;  // [rows, M, nparts, Dv] and [rows, M, nparts, 2] partials
 };
+
+// The visible keys of a 16-query tile as absolute 32-key blocks: the blocks of the kept first
+// tokens that lie before the window (nsink of them, from block 0), then blocks wb0 .. wb1.
+struct WaBlocks { int wb0, nsink, nblocks; };
+EIA_DEV WaBlocks wa_blocks(int pos_first, int pos_last, int window, int keep) {
+  const int lo_min = window > 0 ? max(0, pos_first - window + 1) : 0;
+  const int wb0 = lo_min >> 5;
+  const int nsink = min((min(keep, lo_min) + 31) >> 5, wb0);
+  return WaBlocks{wb0, nsink, nsink + (pos_last >> 5) - wb0 + 1};
+}
+// Key partitions a row really uses: at least four blocks each, so short contexts stay whole
+// whatever the launch's grid.z (the same on both sides of the merge).
+EIA_DEV int wa_parts(int nparts, int nblocks) { return min(nparts, max(1, nblocks >> 2)); }
 
 constexpr int WA_KT = 64;           // keys per tile = lanes of a wave
 constexpr int WA_ACC = 16;          // (map, value column) accumulators per thread
@@ -319,8 +335,9 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
 // ---------------------------------------------------------------------------------------------
 // MFMA form (bf16): v_mfma_f32_16x16x32_bf16, operands straight from the cache into registers.
 //
-// A workgroup of NWV waves owns a tile of 16 queries of one sequence and NWV * HW heads; a wave
-// owns HW heads (HW * P maps) and walks the visible keys in absolute 32-key blocks (a block
+// A workgroup of NWV <= 8 waves owns a tile of 16 queries of one sequence and NWV * HW heads (at
+// most 256 registers per wave, so two waves share a SIMD and one's loads hide behind the other's
+// arithmetic); a wave owns HW heads (HW * P maps) and walks the visible keys in absolute 32-key blocks (a block
 // never straddles a page: block size % 32 == 0), first the blocks of the kept first tokens that
 // lie before the window, then the window's.  Per block and map it forms S^T (keys x queries)
 // as two 16-key tiles whose rows are ordered so that the accumulator registers of a lane --
@@ -332,7 +349,7 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
 // Softmax weights stay fp32: P enters the second product as a bf16 high part plus a bf16
 // remainder, and the normaliser sums the fp32 weights.
 template <int HW, int P, bool TALK, bool SHARE, int ND, int NDV>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 window_attn_mfma_kernel(const WinAttnArgs a) {
   constexpr int MW = HW * P;
   constexpr int NKV = SHARE ? 1 : HW;          // distinct kv heads among this wave's heads
@@ -378,10 +395,10 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   const long row = row0 + (row_ok ? c : 0);
   const int qpos = a.positions[row];
   const int pos_first = a.positions[row0], pos_last = a.positions[row0 + nq - 1];
-  const int lo_min = a.window > 0 ? max(0, pos_first - a.window + 1) : 0;
-  const int wb0 = lo_min >> 5, wb1 = pos_last >> 5;                 // window blocks wb0 .. wb1
-  const int nsink = min((min(a.keep, lo_min) + 31) >> 5, wb0);      // kept-token blocks before wb0
-  const int nblocks = nsink + wb1 - wb0 + 1;
+  const WaBlocks kbs = wa_blocks(pos_first, pos_last, a.window, a.keep);
+  const int wb0 = kbs.wb0, nsink = kbs.nsink, nblocks = kbs.nblocks;
+  const int np = wa_parts(a.nparts, nblocks);
+  if ((int)blockIdx.z >= np) return;                                // (whole workgroup)
 
   // Q^T operands of this wave's maps: column = query c, rows = d 32 s + 8 g .. + 8
   bf16x8 qf[MW][ND];
@@ -415,20 +432,16 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   const int dq = 8 * g;
 
   // with key partitions (decode rows of small batches) this workgroup takes a slice of the blocks
-  const int per = (nblocks + a.nparts - 1) / a.nparts;
+  const int per = (nblocks + np - 1) / np;
   const int b_lo = blockIdx.z * per, b_hi = min(nblocks, b_lo + per);
-  for (int b = b_lo; b < b_hi; ++b) {
-    const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
+  // K operands of one block: every load issued together (addresses clamped, not branched)
+  auto load_k = [&](int b, bf16x8 (&kf)[NKV][P][2][ND]) {
+    const int kb = b < nsink ? b : wb0 + b - nsink;
     const int key0 = kb << 5;
-    const long page = bt[key0 / bs];
-    const int off = key0 % bs;
-    const bf16_t* k0p = kc + (page * bs + off + r0) * krow;
-    f32x4 sc[MW][2];
+    const bf16_t* k0p = kc + ((long)bt[key0 / bs] * bs + key0 % bs + r0) * krow;
 #pragma unroll
     for (int j = 0; j < NKV; ++j) {
       const int kvh = (hs + j * HPK) / rep;
-      // every K operand of this kv head first (addresses clamped, not branched), then the MFMAs
-      bf16x8 kf[P][2][ND];
 #pragma unroll
       for (int pm = 0; pm < P; ++pm)
 #pragma unroll
@@ -437,9 +450,39 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
           const bf16_t* kp = k0p + (kvh * P + pm) * D + (d < D ? d : 0);
           const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kp);
           const bf16x8 kb2 = *reinterpret_cast<const bf16x8*>(kp + 4 * krow);
-          kf[pm][0][s] = d < D ? ka : zero8;
-          kf[pm][1][s] = d < D ? kb2 : zero8;
+          kf[j][pm][0][s] = d < D ? ka : zero8;
+          kf[j][pm][1][s] = d < D ? kb2 : zero8;
         }
+    }
+  };
+  // software pipeline (where the second operand set fits the register budget): block b + 1's
+  // page lookup and K loads are in flight during block b's softmax and second product
+  constexpr bool PIPE = NKV * P * ND <= 4;
+  bf16x8 kf[NKV][P][2][ND], kn[PIPE ? NKV : 1][PIPE ? P : 1][2][PIPE ? ND : 1];
+  if constexpr (PIPE) {
+    if (b_lo < b_hi) load_k(b_lo, kn);
+  }
+  for (int b = b_lo; b < b_hi; ++b) {
+    const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
+    const int key0 = kb << 5;
+    const long page = bt[key0 / bs];
+    const int off = key0 % bs;
+    if constexpr (PIPE) {
+#pragma unroll
+      for (int j = 0; j < NKV; ++j)
+#pragma unroll
+        for (int pm = 0; pm < P; ++pm)
+#pragma unroll
+          for (int s = 0; s < ND; ++s) {
+            kf[j][pm][0][s] = kn[j][pm][0][s];
+            kf[j][pm][1][s] = kn[j][pm][1][s];
+          }
+    } else {
+      load_k(b, kf);
+    }
+    f32x4 sc[MW][2];
+#pragma unroll
+    for (int j = 0; j < NKV; ++j) {
 #pragma unroll
       for (int hh = 0; hh < HPK; ++hh)
 #pragma unroll
@@ -449,8 +492,8 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
           for (int s = 0; s < ND; ++s) {
             if (s < nd) {
-              s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[pm][0][s], qf[m][s], s0, 0, 0, 0);
-              s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[pm][1][s], qf[m][s], s1, 0, 0, 0);
+              s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][pm][0][s], qf[m][s], s0, 0, 0, 0);
+              s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[j][pm][1][s], qf[m][s], s1, 0, 0, 0);
             }
           }
 #pragma unroll
@@ -462,6 +505,9 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
           sc[m][0] = s0;
           sc[m][1] = s1;
         }
+    }
+    if constexpr (PIPE) {
+      if (b + 1 < b_hi) load_k(b + 1, kn);
     }
     // the block's V^T operands are requested before the softmax arithmetic needs them
     bf16x8 vf[NKV][NDV];
@@ -551,7 +597,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   }
   if (!wave_on || !row_ok) return;
   // this lane holds, per map and tile t, value columns 16 t + 4 g + i of query c
-  if (a.nparts > 1) {                               // partials; window_attn_merge finishes the row
+  if (np > 1) {                                     // partials; window_attn_merge finishes the row
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
       const long pr = ((row * M + h0 * P + m) * a.nparts + blockIdx.z);
@@ -625,16 +671,19 @@ window_attn_merge_kernel(const WinAttnArgs a) {
   const int h = blockIdx.y, lane = threadIdx.x;
   bf16_t* out = (bf16_t*)a.out + row * a.ldo + h * Dv;
   if (a.lens && a.lens[row] <= 0) return;           // padding row: the partition kernel wrote zeros
+  const int pos = a.positions[row];
+  const int np = wa_parts(NP, wa_blocks(pos, pos, a.window, a.keep).nblocks);
+  if (np == 1) return;                              // a whole row: already finished and written
   float o[2][2];                                    // [map][column lane, lane + 64]
   for (int pm = 0; pm < P; ++pm) {
     const long pr = (row * M + h * P + pm) * NP;
-    const float mz = lane < NP ? a.part_ml[(pr + lane) * 2] : -1e30f;
-    const float lz = lane < NP ? a.part_ml[(pr + lane) * 2 + 1] : 0.f;
+    const float mz = lane < np ? a.part_ml[(pr + lane) * 2] : -1e30f;
+    const float lz = lane < np ? a.part_ml[(pr + lane) * 2 + 1] : 0.f;
     const float wz = __expf(mz - wave_max(mz));
     const float inv = 1.0f / wave_sum(wz * lz);
     float v0 = 0.f, v1 = 0.f;
 #pragma unroll 4
-    for (int z = 0; z < NP; ++z) {
+    for (int z = 0; z < np; ++z) {
       const float w = __shfl(wz, z, 64);
       if (lane < Dv) v0 += w * a.part_acc[(pr + z) * Dv + lane];
       if (lane + 64 < Dv) v1 += w * a.part_acc[(pr + z) * Dv + lane + 64];
@@ -664,22 +713,19 @@ window_attn_merge_kernel(const WinAttnArgs a) {
 }
 
 // Heads per wave of the MFMA form for (H, P), 0 when the shape runs the scalar form: with head
-// mixing one workgroup must hold every head (H / HW <= 4 waves); without it the heads are
-// spread over grid.y in workgroups of up to four single-head waves.
+// mixing one workgroup must hold every head (H / HW <= 8 waves of one or two heads); without it
+// the heads are spread over grid.y in workgroups of up to four single-head waves.
 static int wa_mfma_hw(int H, int P, int talk) {
   if (!talk) return 1;
   if (P != 1) return 0;
-  if (H <= 4) return 1;
-  if (H <= 8 && H % 2 == 0) return 2;
-  if (H <= 16 && H % 4 == 0) return 4;
+  if (H <= 4 || (H <= 8 && H % 2)) return 1;
+  if (H <= 16 && H % 2 == 0) return 2;
   return 0;
 }
 
 EIA_API int eia_window_attn_mfma_ok(int H, int G, int P, int D, int Dv, int bs, int talk) {
   const int hw = wa_mfma_hw(H, P, talk);
   if (hw == 0 || G < 1 || H % G || D % 8 || D > 128 || Dv % 16 || Dv > 128 || bs % 32) return 0;
-  // four heads of four different kv heads per wave at the large head size would spill
-  if (hw == 4 && (H / G) % 4 != 0 && (D > 64 || Dv > 64)) return 0;
   return 1;
 }
 
@@ -732,10 +778,8 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
   const bool narrow_k = !talk && D <= 64 && Dv > 64;
   if (talk) {
     if (hw == 1) WA_LAUNCH(1, 1, true, true);
-    else if (hw == 2 && share) WA_LAUNCH(2, 1, true, true);
-    else if (hw == 2) WA_LAUNCH(2, 1, true, false);
-    else if (share) WA_LAUNCH(4, 1, true, true);
-    else WA_LAUNCH1(4, 1, true, false, 2, 4);
+    else if (share) WA_LAUNCH(2, 1, true, true);
+    else WA_LAUNCH(2, 1, true, false);
   } else if (P == 2) {
     if (narrow_k) WA_LAUNCH1(1, 2, false, true, 2, 8);
     else WA_LAUNCH(1, 2, false, true);

@@ -60,9 +60,9 @@ def build_work(q_lens: List[int], qblock: int) -> List[int]:
 
 def mfma_ok(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> bool:
     """The MFMA kernel takes bf16 rows with D % 8 == 0, Dv % 16 == 0, both <= 128, pages of a
-    multiple of 32 tokens and, with head mixing, at most 16 heads in 1, 2 or 4 heads per wave
-    (four heads of four different kv heads only up to head size 64); everything else (fp32
-    models too) runs the scalar-FMA kernel."""
+    multiple of 32 tokens and, with head mixing, at most 16 heads (one workgroup of up to eight
+    waves holds them all, one or two heads per wave); everything else (fp32 models too) runs
+    the scalar-FMA kernel."""
     if dtype != torch.bfloat16 or not _MFMA_ENV or not torch.cuda.is_available():
         return False
     return bool(lib().eia_window_attn_mfma_ok(spec.heads, spec.kv_heads, spec.maps, spec.dim,
