@@ -269,7 +269,24 @@ EIA_API int eia_ln_f32in(const float* x, long ldx, const void* w, void* out, lon
 // so a sublayer boundary (output norm, residual add, next input norm) is one pass over the row.
 // A wave owns whole groups and walks them with the same lane-to-column map in both phases, so a
 // lane re-reads only what it wrote and the row needs no barrier.
-template <typename T>
+template <typename T> struct Vec4;
+template <> struct Vec4<bf16_t> { typedef bf16x4 type; };
+template <> struct Vec4<float> { typedef f32x4 type; };
+template <typename T> EIA_DEV f32x4 ld4_f32(const T* p) {
+  const typename Vec4<T>::type v = *reinterpret_cast<const typename Vec4<T>::type*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+template <typename T> EIA_DEV void st4_f32(T* p, f32x4 v) {
+  typename Vec4<T>::type o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = (T)v[i];
+  *reinterpret_cast<typename Vec4<T>::type*>(p) = o;
+}
+EIA_DEV float sumsq4(f32x4 v) { return v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3]; }
+
+// VEC: group size and row strides are multiples of 4, so a lane handles four consecutive columns
+// per step with 8- / 16-byte accesses; otherwise one column per step.
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(256)
 gnorm_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ ypart, int sk,
              long pstride, const T* __restrict__ ybias, const T* __restrict__ w_post,
@@ -294,34 +311,62 @@ gnorm_kernel(const T* __restrict__ y, long ldy, const float* __restrict__ ypart,
     }
     __syncthreads();
   }
-  // the sublayer output at column c: a stored row, or the summed partials
-  auto yval = [&](int c) -> float { return y ? ld_f32<T>(y + row * ldy, c) : ysum[c]; };
+  const T* yr = y ? y + row * ldy : nullptr;
   for (int g = wave; g < NG; g += nw) {
     const int c0 = g * gs;
-    if (y || ypart) {
-      float ss = 0.f;
-      for (int c = lane; c < gs; c += 64) {
-        const float v = yval(c0 + c);
-        ss += v * v;
+    if constexpr (VEC) {
+      if (y || ypart) {
+        float ss = 0.f;
+        for (int c = c0 + 4 * lane; c < c0 + gs; c += 256)
+          ss += sumsq4(y ? ld4_f32<T>(yr + c) : *reinterpret_cast<const f32x4*>(ysum + c));
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+        for (int c = c0 + 4 * lane; c < c0 + gs; c += 256) {
+          const f32x4 v = y ? ld4_f32<T>(yr + c) : *reinterpret_cast<const f32x4*>(ysum + c);
+          f32x4 xv = *reinterpret_cast<f32x4*>(xr + c) + v * inv * ld4_f32<T>(w_post + c);
+          if (add) xv += *reinterpret_cast<const f32x4*>(add + row * (long)W + c);
+          *reinterpret_cast<f32x4*>(xr + c) = xv;
+        }
+      } else if (add) {
+        for (int c = c0 + 4 * lane; c < c0 + gs; c += 256)
+          *reinterpret_cast<f32x4*>(xr + c) += *reinterpret_cast<const f32x4*>(add + row * (long)W + c);
       }
-      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
-      for (int c = lane; c < gs; c += 64)
-        xr[c0 + c] += yval(c0 + c) * inv * ld_f32<T>(w_post, c0 + c);
-    }
-    if (add) {
-      const float* ar = add + row * (long)W + c0;
-      for (int c = lane; c < gs; c += 64) xr[c0 + c] += ar[c];
-    }
-    if (h) {
-      float ss = 0.f;
-      for (int c = lane; c < gs; c += 64) {
-        const float v = xr[c0 + c];
-        ss += v * v;
+      if (h) {
+        float ss = 0.f;
+        for (int c = c0 + 4 * lane; c < c0 + gs; c += 256)
+          ss += sumsq4(*reinterpret_cast<const f32x4*>(xr + c));
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+        for (int c = c0 + 4 * lane; c < c0 + gs; c += 256)
+          st4_f32<T>(h + row * ldh + c,
+                     *reinterpret_cast<const f32x4*>(xr + c) * inv * ld4_f32<T>(w_next + c));
       }
-      const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
-      T* hr = h + row * ldh + c0;
-      for (int c = lane; c < gs; c += 64)
-        st_f32<T>(hr, c, xr[c0 + c] * inv * ld_f32<T>(w_next, c0 + c));
+    } else {
+      // the sublayer output at column c: a stored row, or the summed partials
+      auto yval = [&](int c) -> float { return y ? ld_f32<T>(yr, c) : ysum[c]; };
+      if (y || ypart) {
+        float ss = 0.f;
+        for (int c = lane; c < gs; c += 64) {
+          const float v = yval(c0 + c);
+          ss += v * v;
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+        for (int c = lane; c < gs; c += 64)
+          xr[c0 + c] += yval(c0 + c) * inv * ld_f32<T>(w_post, c0 + c);
+      }
+      if (add) {
+        const float* ar = add + row * (long)W + c0;
+        for (int c = lane; c < gs; c += 64) xr[c0 + c] += ar[c];
+      }
+      if (h) {
+        float ss = 0.f;
+        for (int c = lane; c < gs; c += 64) {
+          const float v = xr[c0 + c];
+          ss += v * v;
+        }
+        const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)gs + eps);
+        T* hr = h + row * ldh + c0;
+        for (int c = lane; c < gs; c += 64)
+          st_f32<T>(hr, c, xr[c0 + c] * inv * ld_f32<T>(w_next, c0 + c));
+      }
     }
   }
 }
@@ -341,14 +386,16 @@ EIA_API int eia_gnorm(const void* y, long ldy, const float* ypart, int sk, const
   const long ps = (long)rows * W;
   const size_t lds = ypart ? sizeof(float) * W : 0;
   if (lds > 64 * 1024) return EIA_UNSUPPORTED;
-  if (is_bf16)
-    hipLaunchKernelGGL((gnorm_kernel<bf16_t>), dim3(rows), dim3(threads), lds, st,
-                       (const bf16_t*)y, ldy, ypart, sk, ps, (const bf16_t*)ybias,
-                       (const bf16_t*)w_post, x, add, (const bf16_t*)w_next, (bf16_t*)h, ldh, eps,
-                       W, NG);
-  else
-    hipLaunchKernelGGL((gnorm_kernel<float>), dim3(rows), dim3(threads), lds, st, (const float*)y,
-                       ldy, ypart, sk, ps, (const float*)ybias, (const float*)w_post, x, add,
-                       (const float*)w_next, (float*)h, ldh, eps, W, NG);
+  const bool vec = (W / NG) % 4 == 0 && ldy % 4 == 0 && ldh % 4 == 0;
+#define GNORM_LAUNCH(TT, VV)                                                                     \
+  hipLaunchKernelGGL((gnorm_kernel<TT, VV>), dim3(rows), dim3(threads), lds, st, (const TT*)y, ldy, \
+                     ypart, sk, ps, (const TT*)ybias, (const TT*)w_post, x, add, (const TT*)w_next, \
+                     (TT*)h, ldh, eps, W, NG)
+  if (is_bf16) {
+    if (vec) GNORM_LAUNCH(bf16_t, true); else GNORM_LAUNCH(bf16_t, false);
+  } else {
+    if (vec) GNORM_LAUNCH(float, true); else GNORM_LAUNCH(float, false);
+  }
+#undef GNORM_LAUNCH
   EIA_LAUNCH_CHECK();
 }

@@ -129,6 +129,7 @@ struct WinAttnArgs {
   const float* lam;                 // [1], epilogue 1
   float eps, post;
   int nparts;                       // MFMA form: key partitions over grid.z (1: none)
+  int raw_bufs;                     // MFMA form with head mixing: raw-score buffers in LDS (1, 2)
   float* part_acc; float* part_ml;  // [rows, M, nparts, Dv] and [rows, M, nparts, 2] partials
 };
 
@@ -141,9 +142,11 @@ EIA_DEV WaBlocks wa_blocks(int pos_first, int pos_last, int window, int keep) {
   const int nsink = min((min(keep, lo_min) + 31) >> 5, wb0);
   return WaBlocks{wb0, nsink, nsink + (pos_last >> 5) - wb0 + 1};
 }
-// Key partitions a row really uses: at least four blocks each, so short contexts stay whole
-// whatever the launch's grid.z (the same on both sides of the merge).
-EIA_DEV int wa_parts(int nparts, int nblocks) { return min(nparts, max(1, nblocks >> 2)); }
+// Key partitions a row really uses: at least two blocks each (a block's dependent chain of
+// loads, products and the exchange is microseconds long, so a lone workgroup should walk few),
+// so short contexts use few partitions whatever the launch's grid.z (the same on both sides of
+// the merge).
+EIA_DEV int wa_parts(int nparts, int nblocks) { return min(nparts, max(1, nblocks >> 1)); }
 
 constexpr int WA_KT = 64;           // keys per tile = lanes of a wave
 constexpr int WA_ACC = 16;          // (map, value column) accumulators per thread
@@ -323,8 +326,8 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
   if (M * Dv > 256 * WA_ACC || lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
-                out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post, 1, nullptr,
-                nullptr};
+                out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post, 1, 2,
+                nullptr, nullptr};
   if (is_bf16)
     hipLaunchKernelGGL((window_attn_kernel<bf16_t>), dim3(n_items), dim3(256), lds, st, a);
   else
@@ -520,7 +523,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
     }
     if constexpr (TALK) {
       // raw scores of every map through LDS: [buffer][map][tile][lane] f32x4
-      f32x4* buf = raw_s + (size_t)(b & 1) * M * 128;
+      f32x4* buf = raw_s + (size_t)(a.raw_bufs == 2 ? (b & 1) : 0) * M * 128;
       if (wave_on) {
 #pragma unroll
         for (int m = 0; m < MW; ++m) {
@@ -544,6 +547,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
           sc[m][1] += tw * r1v;
         }
       }
+      if (a.raw_bufs != 2) __syncthreads();           // one buffer: reads end before it is rewritten
     }
     // mask, running max / sum, P^T operands
     bf16x8 ph[MW], pl[MW];
@@ -750,12 +754,16 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
                 out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post, nparts,
-                part_acc, part_ml};
+                2, part_acc, part_ml};
+  // raw-score buffers of the head-mixing form: two (one barrier per block) while they fit 48 KiB
+  static const int forced_bufs = getenv("EIA_WINDOW_RAW_BUFS") ? atoi(getenv("EIA_WINDOW_RAW_BUFS")) : 0;
+  if (talk) a.raw_bufs = forced_bufs ? forced_bufs : ((size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2);
   const int hw = wa_mfma_hw(H, P, talk != nullptr);
   const int waves_needed = H / hw;
   const int nwv = talk ? waves_needed : (waves_needed < 4 ? waves_needed : 4);
   const int gy = talk ? 1 : (waves_needed + nwv - 1) / nwv;
-  const size_t lds = talk ? (size_t)2 * H * P * 128 * sizeof(f32x4) + sizeof(float) * ((H * H + 3) & ~3) : 0;
+  const size_t lds = talk ? (size_t)a.raw_bufs * H * P * 128 * sizeof(f32x4) +
+                                sizeof(float) * ((H * H + 3) & ~3) : 0;
   if (lds > 128 * 1024) return EIA_UNSUPPORTED;
   const bool share = (H / G) % hw == 0;          // the heads of a wave read one kv head
   const bool big = D > 64 || Dv > 64;

@@ -125,6 +125,14 @@ def group_norm_step(x: torch.Tensor, groups: int, eps: float, y=None,
     T, W = x.shape
     require(W % groups == 0, "group_norm_step: width not divisible by the group count")
     split = isinstance(y, SplitK)
+    if split and use_hip(x) and W % 4:
+        # the kernel sums partials in 16-byte units: other widths (no GEMM of the framework
+        # produces them) take the unfused fp32 sum
+        ys = y.part.sum(0) + (y.bias.float() if y.bias is not None else 0.0)
+        x += _group_rms(ys, groups, eps) * w_post.float()
+        y, split = None, False
+        if add is None and w_next is None:
+            return None
     if not use_hip(x):
         if split:
             y = y.part.sum(0) + (y.bias.float() if y.bias is not None else 0.0)

@@ -73,16 +73,17 @@ def mfma_ok(spec: WindowSpec, dtype: torch.dtype, block_size: int) -> bool:
 def decode_partitions(batch: int, spec: WindowSpec, cus: int = 256) -> int:
     """Key partitions (grid.z) of a decode launch of the MFMA form: a decode row is one
     workgroup (per four heads without head mixing), so small batches split every row's 32-key
-    blocks until about two workgroups per CU exist (a power of two, at most 8, and at least
-    four blocks of a full window per partition); a second kernel merges the partials.  Depends on the
+    blocks until about two workgroups per CU exist (a power of two, at most 16, and at least
+    two blocks of a full window per partition); a second kernel merges the partials.  A row
+    with fewer blocks uses fewer partitions (decided in the kernel).  Depends on the
     batch and the layer's constants only, so a captured decode graph keeps its grid."""
     forced = int(os.environ.get("EIA_WINDOW_DECODE_P", "0"))
     if forced > 0:
         return min(forced, 64)
     wgs = max(1, batch) * (1 if spec.talk is not None else -(-spec.heads // 4))
-    limit = 8
+    limit = 16
     if spec.window > 0:
-        limit = max(1, min(8, ((spec.window + 31) // 32 + 1 + (spec.keep + 31) // 32) // 4))
+        limit = max(1, min(16, ((spec.window + 31) // 32 + 1 + (spec.keep + 31) // 32) // 2))
     p = 1
     while p * 2 <= limit and wgs * p * 2 <= 2 * cus:
         p *= 2
@@ -112,6 +113,10 @@ def qk_norm_cache(fused, q_off: int, k_off: int, v_off: int, mq: int, mk: int,
     split = isinstance(fused, SplitK)
     if split and not fused.part.is_cuda:            # CPU path: the plain fp32 sum
         fused = fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
+        split = False
+    elif split and fused.N % 4:                     # the kernel sums partials in 16-byte units
+        fused = (fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
+                 ).to(k_cache.dtype)
         split = False
     if not split:
         T = fused.shape[0]
