@@ -48,11 +48,19 @@ static_assert(KLANE == 8 || KLANE == 32, "EIA_GEMM_KLANE must be 8 or 32");
 // MODE_SWIGLU_SPLIT: the SwiGLU pairing over a K range split across grid.y -- fp32 gate and
 // up partials [sk][M][2I] (gate at n, up at I + n), finished by eia_splitk_swiglu.  For gate/up
 // widths too narrow to fill the chip with whole-K pair tiles (Llama-70B at TP 8: 224 tiles).
-enum Mode : int { MODE_BF16 = 0, MODE_F32_SPLIT = 1, MODE_SWIGLU = 2, MODE_SWIGLU_SPLIT = 3 };
+// MODE_GEGLU: the SwiGLU pairing with the tanh form of GELU on the gate (its split-K form is
+// MODE_SWIGLU_SPLIT, whose partials carry no activation yet).
+enum Mode : int { MODE_BF16 = 0, MODE_F32_SPLIT = 1, MODE_SWIGLU = 2, MODE_SWIGLU_SPLIT = 3,
+                  MODE_GEGLU = 4 };
 
-__host__ __device__ inline bool swiglu_pairing(int mode) { return mode == MODE_SWIGLU || mode == MODE_SWIGLU_SPLIT; }
+__host__ __device__ inline bool swiglu_pairing(int mode) {
+  return mode == MODE_SWIGLU || mode == MODE_SWIGLU_SPLIT || mode == MODE_GEGLU;
+}
 
 EIA_DEV float silu(float x) { return __fdividef(x, 1.f + __expf(-x)); }
+EIA_DEV float gelu_tanh(float x) {
+  return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
 
 // Weight-stream load.  Non-temporal loads (EIA_GEMM_NT) measured 1.7x SLOWER on this box for
 // back-to-back decode replays (guide: MI355X_MICROARCH "nt-weights" -- nt gives up what a
@@ -84,7 +92,7 @@ EIA_DEV void store_tile(const f32x4 (&acc)[NT][MT], int mode, void* __restrict__
     }
     return;
   }
-  if (NT == 2 && mode == MODE_SWIGLU) {
+  if (NT == 2 && (mode == MODE_SWIGLU || mode == MODE_GEGLU)) {
     bf16_t* o = reinterpret_cast<bf16_t*>(out);
     const int n = nbase + 4 * g;
 #pragma unroll
@@ -92,8 +100,13 @@ EIA_DEV void store_tile(const f32x4 (&acc)[NT][MT], int mode, void* __restrict__
       const int row = m * 16 + r;
       if (row < Mc) {
         bf16x4 v;
+        if (mode == MODE_GEGLU) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = f2bf(silu(acc[0][m][i]) * acc[NT - 1][m][i]);
+          for (int i = 0; i < 4; ++i) v[i] = f2bf(gelu_tanh(acc[0][m][i]) * acc[NT - 1][m][i]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) v[i] = f2bf(silu(acc[0][m][i]) * acc[NT - 1][m][i]);
+        }
         *reinterpret_cast<bf16x4*>(o + (orow0 + row) * ldo + n) = v;
       }
     }
@@ -902,7 +915,8 @@ int check_shape(int N, int K, int sk, int mode, int cfg) {
   if ((cfg & 128) && ((cfg & 32) || !(cfg & 16) || !(cfg & 2) || ((cfg >> 2) & 3) == 3))
     return EIA_BAD_SHAPE;                                                // LDS-DMA ring
   if (swiglu_pairing(mode)) {
-    if (nt != 2 || (mode == MODE_SWIGLU && sk != 1) || N % 2 != 0 || (N / 2) % (waves * 16) != 0)
+    if (nt != 2 || ((mode == MODE_SWIGLU || mode == MODE_GEGLU) && sk != 1) || N % 2 != 0 ||
+        (N / 2) % (waves * 16) != 0)
       return EIA_BAD_SHAPE;
   } else if (N % (waves * nt * 16) != 0) {
     return EIA_BAD_SHAPE;
@@ -917,7 +931,8 @@ int check_shape(int N, int K, int sk, int mode, int cfg) {
 // mode 1: out fp32 partial slabs [sk][M][N] (reduce with eia_splitk_reduce / _add_rmsnorm)
 // mode 2: SwiGLU: W = merged [gate; up] (N = 2I rows), out bf16 [M][ldo] = silu(gate) * up
 // mode 3: SwiGLU pairing, K split over sk: out fp32 [sk][M][2I] (gate n, up I + n), finished by
-//         eia_splitk_swiglu
+//         eia_splitk_swiglu (or eia_splitk_act_and_mul for another activation)
+// mode 4: as mode 2 with gelu_tanh(gate) * up
 // cfg: bit0 -> two 16-row W tiles per wave (else one), bit1 -> 4 waves per workgroup (else 2),
 // bits 2-3 -> W pipeline stages - 2 (2..4), bit 4 -> 128-deep K chunks (else 256),
 // bit 5 -> extra X-loader wave (with bits 1 and 4), bit 6 -> tile-packed W (ldw must be K),

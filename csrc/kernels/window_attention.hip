@@ -756,8 +756,7 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
                 out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post, nparts,
                 2, part_acc, part_ml};
   // raw-score buffers of the head-mixing form: two (one barrier per block) while they fit 48 KiB
-  static const int forced_bufs = getenv("EIA_WINDOW_RAW_BUFS") ? atoi(getenv("EIA_WINDOW_RAW_BUFS")) : 0;
-  if (talk) a.raw_bufs = forced_bufs ? forced_bufs : ((size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2);
+  if (talk) a.raw_bufs = (size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2;
   const int hw = wa_mfma_hw(H, P, talk != nullptr);
   const int waves_needed = H / hw;
   const int nwv = talk ? waves_needed : (waves_needed < 4 ? waves_needed : 4);

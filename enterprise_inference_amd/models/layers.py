@@ -84,14 +84,16 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
     def forward_act_and_mul(self, x, act: str = "silu"):
         """act(x Wg^T) * (x Wu^T) for a [gate; up] merged projection.
 
-        Decode-sized batches run the fused SwiGLU GEMM (K7: the 2I-wide
-        intermediate never reaches HBM); prompt-sized ones hipBLASLt (TunableOp picks, 1.5-1.6
+        Decode-sized batches run the fused gated-activation GEMM (K7, SiLU or the tanh form of
+        GELU in its epilogue: the 2I-wide intermediate never reaches HBM); prompt-sized ones hipBLASLt (TunableOp picks, 1.5-1.6
         PFLOP/s) + the act_and_mul kernel -- a hand MFMA form with the epilogue fused reached
         1.2 PFLOP/s and lost in the prefill step, so it was removed (docs/performance.md).
         """
-        if act == "silu" and self.bias is None and len(self.out_sizes) == 2 and \
+        fused = "silu" if act == "silu" else "gelu_tanh" if act in (
+            "gelu_tanh", "gelu_pytorch_tanh", "gelu_new") else None
+        if fused and self.bias is None and len(self.out_sizes) == 2 and \
                 x.dim() == 2 and gemm.skinny_ok(x, self.weight, swiglu=True):
-            return gemm.swiglu_gemm(x, self.weight)
+            return gemm.swiglu_gemm(x, self.weight, act=fused)
         from ..ops import activation
         if self.bias is None and x.dim() == 2:
             # other activations: a decode-sized GEMM's split-K partials are summed inside the

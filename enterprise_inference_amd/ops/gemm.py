@@ -33,7 +33,7 @@ TUNING_FILE = resolve("gemm_tuning.json", os.path.join(_HERE, "gemm_tuning.json"
 PREFILL_TUNING_FILE = resolve("tunableop_mi355x.csv", os.path.join(_HERE, "tunableop_mi355x.csv"),
                               "EIA_PREFILL_GEMM_TUNING")
 
-MODE_BF16, MODE_SPLIT, MODE_SWIGLU, MODE_SWIGLU_SPLIT = 0, 1, 2, 3
+MODE_BF16, MODE_SPLIT, MODE_SWIGLU, MODE_SWIGLU_SPLIT, MODE_GEGLU = 0, 1, 2, 3, 4
 # kernel configs: bit0 -> 2 W tiles (32 rows) per wave, bit1 -> 4 waves per workgroup
 # bit0 NT=2, bit1 WAVES=4, bits2-3 pipeline stages-2, bit4 128-deep K chunks (else 256)
 # bit5: an extra wave stages X into LDS (4 compute waves, KC 128): 50, 51, 54, 55, 58, 59
@@ -442,10 +442,14 @@ def linear_f32(x: torch.Tensor, w: torch.Tensor) -> Optional[torch.Tensor]:
 
 
 def swiglu_gemm(x: torch.Tensor, w_gate_up: torch.Tensor, cfg: Optional[int] = None,
-                sk: Optional[int] = None) -> torch.Tensor:
-    """silu(x Wg^T) * (x Wu^T) with W = [gate; up] stacked on dim 0 (K7).  ``sk`` > 1 splits K
-    over grid.y (fp32 gate / up partials, finished by one small SwiGLU-reduce launch): for
-    gate/up widths whose whole-K pair tiles cannot fill the chip (Llama-70B at TP 8: 224)."""
+                sk: Optional[int] = None, act: str = "silu") -> torch.Tensor:
+    """act(x Wg^T) * (x Wu^T) with W = [gate; up] stacked on dim 0 (K7); ``act`` is ``silu`` or
+    ``gelu_tanh``.  ``sk`` > 1 splits K over grid.y (fp32 gate / up partials, finished by one
+    small gated-activation reduce launch): for gate/up widths whose whole-K pair tiles cannot
+    fill the chip (Llama-70B at TP 8: 224)."""
+    if act not in ("silu", "gelu_tanh"):
+        raise ValueError("swiglu_gemm: act must be silu or gelu_tanh")
+    gelu = act != "silu"
     M, K = x.shape
     N = w_gate_up.shape[0]
     if cfg is None:
@@ -458,13 +462,18 @@ def swiglu_gemm(x: torch.Tensor, w_gate_up: torch.Tensor, cfg: Optional[int] = N
     out = torch.empty(M, N // 2, dtype=torch.bfloat16, device=x.device)
     if sk == 1:
         check(lib().eia_gemm_skinny(ptr(x), x.stride(0), ptr(w_gate_up), w_gate_up.stride(0),
-                                    None, ptr(out), out.stride(0), M, N, K, 1, MODE_SWIGLU, cfg,
-                                    stream(x)), "gemm_skinny_swiglu")
+                                    None, ptr(out), out.stride(0), M, N, K, 1,
+                                    MODE_GEGLU if gelu else MODE_SWIGLU, cfg, stream(x)),
+              "gemm_skinny_swiglu")
         return out
     part = torch.empty(sk, M, N, dtype=torch.float32, device=x.device)
     check(lib().eia_gemm_skinny(ptr(x), x.stride(0), ptr(w_gate_up), w_gate_up.stride(0), None,
                                 ptr(part), N, M, N, K, sk, MODE_SWIGLU_SPLIT, cfg, stream(x)),
           "gemm_skinny_swiglu_split")
+    if gelu:
+        check(lib().eia_splitk_act_and_mul(ptr(part), sk, M, N // 2, ptr(out), out.stride(0), 1,
+                                           stream(x)), "splitk_act_and_mul")
+        return out
     check(lib().eia_splitk_swiglu(ptr(part), sk, M, N // 2, ptr(out), out.stride(0), stream(x)),
           "splitk_swiglu")
     return out

@@ -79,6 +79,23 @@ def test_generate_graph_decode_config_c():
     K.case_generate("cuda", torch.bfloat16, C.config_c, expect_graphs=True)
 
 
+@pytest.mark.parametrize("shape", [(1, 2048, 1024), (32, 4096, 1024), (7, 512, 256), (48, 8192, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_gated_gelu_gemm(shape):
+    """The decode-sized [gate; up] GEMM with the tanh form of GELU in its epilogue (or, where it
+    splits K, in the reduce kernel) against the plain fp32 product."""
+    from enterprise_inference_amd.models.layers import MergedColumnParallelLinear
+    M, I, K = shape
+    g = torch.Generator().manual_seed(M + I)
+    lin = MergedColumnParallelLinear(K, [I, I], dtype=torch.bfloat16, device="cuda")
+    lin.weight.data.copy_((torch.randn(2 * I, K, generator=g) * K ** -0.5).to(torch.bfloat16))
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    got = lin.forward_act_and_mul(x, "gelu_tanh").float().cpu()
+    y = x.float().cpu() @ lin.weight.float().cpu().t()
+    want = torch.nn.functional.gelu(y[:, :I], approximate="tanh") * y[:, I:]
+    assert torch.allclose(got, want, atol=2e-2, rtol=2e-2), float((got - want).abs().max())
+
+
 def test_native_library_loaded():
     from enterprise_inference_amd import _native
     lib = _native.kernels()
