@@ -149,6 +149,7 @@ EIA_DEV WaBlocks wa_blocks(int pos_first, int pos_last, int window, int keep) {
 EIA_DEV int wa_parts(int nparts, int nblocks) { return min(nparts, max(1, nblocks >> 1)); }
 
 constexpr int WA_KT = 64;           // keys per tile = lanes of a wave
+constexpr int WA_PAGES = 256;       // MFMA form: block -> page entries kept in LDS
 constexpr int WA_ACC = 16;          // (map, value column) accumulators per thread
 
 // Scalar-FMA form (fp32 models; bf16 shapes the MFMA form does not take).  One workgroup of four
@@ -437,11 +438,22 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   // with key partitions (decode rows of small batches) this workgroup takes a slice of the blocks
   const int per = (nblocks + np - 1) / np;
   const int b_lo = blockIdx.z * per, b_hi = min(nblocks, b_lo + per);
+  // the pages of this workgroup's blocks, looked up once (the block loop then has no dependent
+  // global load in front of its operand addresses); blocks past the table's size look up directly
+  __shared__ int page_s[WA_PAGES];
+  for (int i = threadIdx.x; i < min(b_hi - b_lo, WA_PAGES); i += blockDim.x) {
+    const int bb = b_lo + i;
+    page_s[i] = bt[((bb < nsink ? bb : wb0 + bb - nsink) << 5) / bs];
+  }
+  __syncthreads();
+  auto page_of = [&](int b, int key0) -> long {
+    return b - b_lo < WA_PAGES ? page_s[b - b_lo] : bt[key0 / bs];
+  };
   // K operands of one block: every load issued together (addresses clamped, not branched)
   auto load_k = [&](int b, bf16x8 (&kf)[NKV][P][2][ND]) {
     const int kb = b < nsink ? b : wb0 + b - nsink;
     const int key0 = kb << 5;
-    const bf16_t* k0p = kc + ((long)bt[key0 / bs] * bs + key0 % bs + r0) * krow;
+    const bf16_t* k0p = kc + (page_of(b, key0) * bs + key0 % bs + r0) * krow;
 #pragma unroll
     for (int j = 0; j < NKV; ++j) {
       const int kvh = (hs + j * HPK) / rep;
@@ -468,7 +480,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   for (int b = b_lo; b < b_hi; ++b) {
     const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
     const int key0 = kb << 5;
-    const long page = bt[key0 / bs];
+    const long page = page_of(b, key0);
     const int off = key0 % bs;
     if constexpr (PIPE) {
 #pragma unroll
